@@ -549,8 +549,19 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
                          const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page, int tokens,
                          int heads, int kv_heads, int d, int dv, float eps, int f32, mv_stream_t stream);
 
+/* Rows of qk are [heads x d | kv_heads x d] fp32, one projection's output.  Queries: q += q_bias (NULL: none), then
+ * the first `rot` dimensions of each head rotated by angle pos * inv_freq[i] (fp64 table of rot/2 entries; adjacent:
+ * dimension 2i with 2i+1, else i with i + rot/2), in place.  Keys: k += k_bias; the key as it then stands goes to
+ * v_cache (attention whose values are its unrotated keys), its rotated form to k_cache, both [pages, page, kv_heads, d]. */
+int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* k_bias, void* k_cache, void* v_cache,
+                       const double* inv_freq, const int32_t* tok_row, const int32_t* tok_pos,
+                       const int32_t* block_table, int bt_stride, int page, int tokens, int heads, int kv_heads, int d,
+                       int rot, int adjacent, int f32, mv_stream_t stream);
+
 /* out[t, h*dv ..] = softmax_j( q_t . k_j * scale - slopes[h] * (pos - j) ) v_j over pos - window < j <= pos
- * from the pages (the step's own keys must already be stored).  dv <= 256.  With a chunk table (chunks > 0:
+ * from the pages (the step's own keys must already be stored).  dv <= 256.  keep_first > 0: positions below it
+ * stay visible when the window has passed them, at their true positions.  sinks (fp32 [heads] or NULL): exp(sinks[h])
+ * is one more term of the softmax's denominator, unscaled, with no value.  slopes NULL: no distance penalty.  With a chunk table (chunks > 0:
  * rows of more than max_len tokens cut into runs of up to 64, as for mv_scan_chunked; row_len per row), bf16
  * and a head shape the tiled kernel is built for - (d, dv) in (32,32) (64,64) (96,96) (128,128) (128,64)
  * (64,128), 64-token pages - those rows run on the matrix cores, a workgroup per (chunk, head): q.k in bf16
@@ -560,7 +571,7 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
-                   int chunks, int max_len, mv_stream_t stream);
+                   int chunks, int max_len, int keep_first, const float* sinks, mv_stream_t stream);
 
 /* ---- further row-wise steps of fp32-stream stacks (stream_ops.hip) ---------------------------------- */
 
@@ -590,6 +601,22 @@ int mv_gelu_gate_rows(const float* a, int64_t lda, const void* table, int64_t ld
                       int vocab, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
 /* out = act( silu(a[:, :n]) * a[:, n:2n] ). */
 int mv_silu_mul(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+/* out = act( f(a[:, :n]) * a[:, n:2n] ): kind 0 f = SiLU, 1 f = GELU in its tanh form; kind 2 the clamped gate,
+ * g = min(a[:, :n], limit), u = clamp(a[:, n:2n], -limit, limit), out = act( g * sigmoid(slope * g) * (u + 1) ). */
+int mv_gated_act(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int kind, float limit,
+                 float slope, int f32, mv_stream_t stream);
+/* x[r,:] = table[ids[r],:] * scale + pairs[j,:] (fp32), j = (prev[r] * mul_prev + ids[r] * mul_cur) mod buckets, or
+ * j = buckets (the table's extra last row) where prev[r] < 0: the token has no predecessor.  Tables in the
+ * activation type, `pairs` [buckets + 1, n]. */
+int mv_embed_pair(const void* table, const void* pairs, const int32_t* ids, const int32_t* prev, float* x, int64_t ldx,
+                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale, int f32,
+                  mv_stream_t stream);
+/* x += y1 (+ y2) (y1 == NULL: x as it is); w != NULL: h = act( x / sqrt(mean(x^2) + eps) * w ). */
+int mv_add_rmsnorm(const float* y1, int64_t ld1, const float* y2, int64_t ld2, float* x, int64_t ldx, const float* w,
+                   float eps, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
+/* out[r,:] = act( x[idx[r],:] / sqrt(mean(.^2) + eps) * (offset + w) ); idx == NULL: row r itself. */
+int mv_rmsnorm_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, float eps, float offset,
+                      void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
 /* out = act( a * sigmoid(g) ); g == NULL: act(a). */
 int mv_sigmoid_gate(const float* a, int64_t lda, const float* g, int64_t ldg, void* out, int64_t ldo, int rows, int n,
                     int f32, mv_stream_t stream);
@@ -650,15 +677,23 @@ int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out
 int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float* w_shared_gate, int32_t* ids,
                  float* weights, float* shared_gate, int tokens, int n, int experts, int top, int f32,
                  mv_stream_t stream);
+/* scores = softmax over all `experts` router outputs of W_router h (fp32); the `top` largest of score + correction
+ * (NULL: none; ties to the lower index) are chosen; weights = score / (sum of the chosen scores + sum_floor) * scale. */
+int mv_moe_route_scored(const void* h, int64_t ldh, const float* w_router, const float* correction, int32_t* ids,
+                        float* weights, int tokens, int n, int experts, int top, float scale, float sum_floor, int f32,
+                        mv_stream_t stream);
 /* (token, choice) pairs sorted by expert: seg [experts + 1], order [pairs] (pair in each row), place [pairs]. */
 int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place, int pairs, int experts,
                 mv_stream_t stream);
 /* s_t = sum_k weights[t,k] * expert_out[place[t*top+k]] (+ shared_gate[t] * shared_out[t]).  norm_w == NULL: y = s.
- * Else y is the residual stream: y += tanh(norm_alpha s) norm_w + norm_b, and h (optional) = act(y). */
+ * Else y is the residual stream: y += tanh(norm_alpha s) norm_w + norm_b, and h (optional) = act(y).
+ * ids != NULL: a choice ids[t*top+k] >= first_pass has no expert row; it adds weights[t,k] * pass[t,:] (activation
+ * type, row stride ldp): an expert that hands its input through. */
 int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
                    const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy,
                    const float* norm_w, const float* norm_b, const float* norm_alpha, void* h, int64_t ldh, int tokens,
-                   int n, int top, int f32, mv_stream_t stream);
+                   int n, int top, int f32, const int32_t* ids, int first_pass, const void* pass, int64_t ldp,
+                   mv_stream_t stream);
 
 #ifdef __cplusplus
 }

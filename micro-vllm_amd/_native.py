@@ -108,7 +108,13 @@ PROTOTYPES = {
     "mv_gated_group_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P]),
     "mv_qk_unitnorm_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
     "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I,
-                            _P, _P, _P, _I, _I, _P]),
+                            _P, _P, _P, _I, _I, _I, _P, _P]),
+    "mv_qk_rotary_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "mv_gated_act": (_I, [_P, _L, _P, _L, _I, _I, _I, _F, _F, _I, _P]),
+    "mv_embed_pair": (_I, [_P, _P, _P, _P, _P, _L, _I, _I, _I, _L, _L, _L, _F, _I, _P]),
+    "mv_add_rmsnorm": (_I, [_P, _L, _P, _L, _P, _L, _P, _F, _P, _L, _I, _I, _I, _P]),
+    "mv_rmsnorm_gather": (_I, [_P, _L, _P, _P, _F, _F, _P, _L, _I, _I, _I, _P]),
+    "mv_moe_route_scored": (_I, [_P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _F, _F, _I, _P]),
     "mv_dyt_shift": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _P]),
     "mv_dyt_gather": (_I, [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P]),
     "mv_dyt_residual": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _I, _I, _I, _P]),
@@ -128,7 +134,8 @@ PROTOTYPES = {
                             _P]),
     "mv_moe_route": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mv_moe_plan": (_I, [_P, _P, _P, _P, _I, _I, _P]),
-    "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P]),
+    "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P, _I, _P, _L,
+                            _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),

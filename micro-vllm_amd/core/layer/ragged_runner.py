@@ -35,6 +35,19 @@ Per layer (Fagunex; norms are Dynamic Tanh, before and after each sublayer):
             in one launch
   side      gate projection of x -> gelu_tanh * slice of the second embedding -> projection ->
             x += unit-RMS * weight
+
+Per layer (Nesisun; both sublayers of a layer read ONE RMS norm and enter the stream together):
+  embedding table row * scale + row of the pair-hashed table (the token before each token comes with the step)
+  attention ONE projection of h gives q | k (| gate | up of a dense feed-forward) -> biases, rotation of adjacent pairs,
+            the rotated key into the key page and the key as projected into the value page (the values ARE the
+            unrotated keys) -> softmax attention over the window and the kept first positions with a sink in the
+            denominator, written beside the feed-forward's activations
+  dense     gelu_tanh(gate) * up lands next to the attention output; ONE projection over [attention | activations]
+            with [W_o | W_down] gives mixer + feed-forward
+  moe       router (fp32 softmax over all outputs, correction for the choice only, renormalised weights) -> pairs
+            sorted by expert -> gate|up by segment -> clamped gate -> down by segment -> weighted sum, a choice of
+            a pass-through expert adding h itself; W_o separately
+  then      x += both, and the NEXT layer's norm of the new x, in one launch
 """
 import logging
 from typing import Dict, List, Optional
@@ -42,6 +55,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ...kernel import ragged_ops as ops
+from ...models.nesisun import GATE_SLOPE, WEIGHT_SUM_FLOOR
 from ...models.pagazen import mamba2_sizes
 from ..state_cache import HybridCacheManager, RaggedStep
 
@@ -72,6 +86,7 @@ class RaggedRunner:
         # a layer RUN = (layer whose tensors it uses, its description); every run has a cache / state of its own
         self.runs = cfg.layer_runs()
         self.sandwich = cfg.architecture == "Fagunex"     # Dynamic Tanh before and after each sublayer
+        self.parallel_prenorm = cfg.architecture == "Nesisun"   # one RMS norm feeds mixer and feed-forward alike
         for wi, layer in self.runs:
             if wi not in self._w:
                 self._w[wi] = self._prepare_layer(wi, layer)
@@ -79,6 +94,9 @@ class RaggedRunner:
         if self.sandwich:
             self.final_norm = self._dyt_norm("final.norm")
             self.side_embed = self._act(model.get("side.embed")) if cfg.side_dim else None
+        elif self.parallel_prenorm:
+            self.final_norm = self._small(model.get("final.norm"))
+            self.pair_embed = self._act(model.get("bigram"))
         else:
             self.final_norm = self._small(model.get("final.norm"))
         self.head = self._linear(model.get("head"))
@@ -109,6 +127,8 @@ class RaggedRunner:
     def _prepare_layer(self, i: int, layer: dict) -> dict:
         if self.sandwich:
             return self._prepare_fagunex(i, layer)
+        if self.parallel_prenorm:
+            return self._prepare_nesisun(i, layer)
         g, p, m = self.model.get, f"l{i}.", layer["mixer"]
         w = {"norm1": self._small(g(p + "norm1"))}
         if layer["type"] == "mamba2":
@@ -176,6 +196,30 @@ class RaggedRunner:
                      side_norm=self._small(g(p + "side.norm")), side_off=i * cfg.side_dim)
         return w
 
+    def _prepare_nesisun(self, i: int, layer: dict) -> dict:
+        g, p, m = self.model.get, f"l{i}.", layer["mixer"]
+        rot = int(m["rot"]["dims"])
+        inv_freq = float(m["rot"]["base"]) ** (-2.0 * torch.arange(max(rot // 2, 1), dtype=torch.float64) / max(rot, 1))
+        w = {"norm1": self._small(g(p + "norm1")), "q_b": self._small(g(p + "mix.q.b")),
+             "k_b": self._small(g(p + "mix.k.b")), "sink": self._small(g(p + "mix.sink")),
+             "inv_freq": inv_freq.to(self.device)}
+        mlp = layer.get("mlp")
+        if mlp and mlp["kind"] == "dense":
+            # both sublayers read the same h and their outputs are summed: one projection in (q | k | gate | up),
+            # one out ([W_o | W_down] over [attention output | activations])
+            w.update(w_in=self._linear(g(p + "mix.q"), g(p + "mix.k"), g(p + "mlp.gate"), g(p + "mlp.up")),
+                     w_out=self._linear(torch.cat([g(p + "mix.o"), g(p + "mlp.down")], dim=1)))
+        else:
+            w.update(w_in=self._linear(g(p + "mix.q"), g(p + "mix.k")), w_out=self._linear(g(p + "mix.o")))
+        if mlp and mlp["kind"] == "moe":
+            E = int(mlp["router"]["experts"])
+            w.update(router=self._small(g(p + "mlp.router")), correction=self._small(g(p + "mlp.correction")))
+            if E:
+                w.update(e_gu=self._stacked([torch.cat([g(p + f"mlp.e{e}.gate"), g(p + f"mlp.e{e}.up")], dim=0)
+                                             for e in range(E)]),
+                         e_down=self._stacked([g(p + f"mlp.e{e}.down") for e in range(E)]))
+        return w
+
     # ------------------------------------------------------------------ cache geometry
     def cache_layout(self):
         """(kv_layers, state_layers) for HybridCacheManager: what every layer RUN keeps per sequence."""
@@ -185,6 +229,8 @@ class RaggedRunner:
             if layer["type"] == "mamba2":
                 s = mamba2_sizes(m)
                 state[i] = {"conv": (max(s["taps"] - 1, 0), s["conv_ch"]), "ssm": (s["heads"], s["n"], s["p"])}
+            elif layer["type"] == "attention":
+                kv[i] = (int(m["kv_heads"]), int(m["dim"]), int(m["dim"]))   # rotated key | the key as projected = value
             elif layer["type"] == "hgrn2":
                 state[i] = {"shift": (self.width,), "gated": (int(m["heads"]), int(m["dim"]), int(m["vdim"]))}
             elif layer["type"] in ("latent_attention", "latent_attention_2"):
@@ -333,7 +379,18 @@ class RaggedRunner:
     def _run(self, step: RaggedStep, cache: HybridCacheManager, want, residuals) -> torch.Tensor:
         cfg, T = self.cfg, step.tokens
         x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
-        if self.sandwich:
+        if self.parallel_prenorm:
+            ops.embed_pair(self.embed, self.pair_embed, step.ids, step.tok_prev, x, cfg.embed_scale, cfg.pair_buckets,
+                           cfg.pair_mul_prev, cfg.pair_mul_cur)
+            ops.add_rmsnorm(x, w=self._w[self.runs[0][0]]["norm1"], eps=cfg.eps, h=h)
+            for li, (wi, layer) in enumerate(self.runs):
+                y1, y2 = self._nesisun_layer(li, self._w[wi], layer, h, step, cache)
+                # both sublayers enter the stream; the next layer's norm of the new x comes out of the same launch
+                nxt = self._w[self.runs[li + 1][0]]["norm1"] if li + 1 < len(self.runs) else None
+                ops.add_rmsnorm(x, y1, y2, w=nxt, eps=cfg.eps, h=None if nxt is None else h)
+                if residuals is not None:
+                    residuals.append(x.clone())
+        elif self.sandwich:
             ops.embed_scaled(self.embed, step.ids, 1.0, x, h)
             for li, (wi, layer) in enumerate(self.runs):
                 self._fagunex_layer(li, self._w[wi], layer, x, h, step, cache)
@@ -363,12 +420,55 @@ class RaggedRunner:
             return self._f32buf(0, self.vocab_size)
         if self.sandwich:
             ops.dyt_gather(x, want, self.final_norm, normed)
+        elif self.parallel_prenorm:
+            ops.rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
         else:
             ops.offset_rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
         logits = self.head(normed, self._f32buf(rows, self.vocab_size))
         if getattr(cfg, "logit_softcap", None):
             ops.softcap_(logits, cfg.logit_softcap)
         return logits
+
+    # ------------------------------------------------------------------ Nesisun layers
+    def _nesisun_layer(self, li, w, layer, h, step: RaggedStep, cache: HybridCacheManager):
+        """Mixer and feed-forward of one layer run on the normed input h: returns their outputs (fp32; the second
+        is None where one projection has already summed them, or where there is no feed-forward)."""
+        T, m, mlp = step.tokens, layer["mixer"], layer.get("mlp")
+        H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
+        dense = bool(mlp) and mlp["kind"] == "dense"
+        ff = int(mlp["ff"]) if dense else 0
+        proj = w["w_in"](h, self._f32buf(T, w["w_in"].n))          # [q | k (| gate | up)]
+        qk = proj[:, :(H + G) * d]
+        kc, vc = cache.k_caches[li], cache.v_caches[li]
+        ops.qk_rotary_store(qk, w["q_b"], w["k_b"], kc, vc, w["inv_freq"], step, H, G, d, int(m["rot"]["dims"]),
+                            adjacent=True)
+        cat = self._actbuf(T, H * d + ff)                          # [attention output | activations]
+        ops.window_attn(qk, kc, vc, cat[:, :H * d], step, None, H, G, d, d, float(m["scale"]), int(m["mask"]["size"]),
+                        tiled=self.tiled_attn, keep_first=int(m["mask"].get("keep_first", 0)), sinks=w["sink"])
+        if dense:
+            ops.gated_act(proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH)
+        y1 = w["w_out"](cat, self._f32buf(T, self.width))
+        if not mlp or dense:
+            return y1, None
+        return y1, self._routed_with_pass(w, mlp, h, T)
+
+    def _routed_with_pass(self, w, mlp, h, T):
+        r = mlp["router"]
+        E, n_pass, top, ff = int(r["experts"]), int(r.get("identity", 0)), int(r["top"]), int(mlp["expert"]["ff"])
+        ids = self._i32buf(T * top).view(T, top)
+        wts = self._f32buf(T, top)
+        ops.moe_route_scored(h, w["router"], w["correction"], ids, wts, float(r.get("scale", 1.0)), WEIGHT_SUM_FLOOR)
+        seg, order, place = self._i32buf(E + n_pass + 1), self._i32buf(T * top), self._i32buf(T * top)
+        ops.moe_plan(ids, seg, order, place, E + n_pass)
+        down = self._f32buf(T * top, self.width)
+        if E:
+            gu = ops.linear_segments(h, w["e_gu"], self._f32buf(T * top, 2 * ff), seg[:E + 1], order, top, T)
+            act = self._actbuf(T * top, ff)
+            ops.gated_act(gu, act, ops.GATE_CLAMPED, float(mlp["expert"]["limit"]), GATE_SLOPE)
+            ops.linear_segments(act, w["e_down"], down, seg[:E + 1], None, 1, T)
+        y = self._f32buf(T, self.width)
+        ops.moe_combine(down, place, wts, None, None, y, ids=ids.view(-1), first_pass=E, passed=h)
+        return y
 
     # ------------------------------------------------------------------ Fagunex layers
     def _i32buf(self, count):

@@ -8,8 +8,9 @@ free lists when it ends.  Nothing is cleared on reuse: a page row is written bef
 and the kernels take the state of a sequence that has no tokens yet as zero.
 
 `plan()` lays one step out for the kernels (csrc/seq_mix.hip): tokens of all rows back to back with
-each token's row and position, per row its first token, length, tokens held before, slot, and its
-row of the block table - one pinned staging buffer and one host-to-device copy per step.
+each token's row, position and predecessor (a sequence's last token is kept on the host between steps,
+for embeddings that look at pairs of tokens), per row its first token, length, tokens held before, slot,
+and its row of the block table - one pinned staging buffer and one host-to-device copy per step.
 """
 import collections
 from dataclasses import dataclass
@@ -26,6 +27,7 @@ class RaggedStep:
     ids: torch.Tensor          # int32 [T]
     tok_row: torch.Tensor      # int32 [T]
     tok_pos: torch.Tensor      # int32 [T]
+    tok_prev: torch.Tensor     # int32 [T] the token before each token in its sequence, -1 at position 0
     row_start: torch.Tensor    # int32 [B]
     row_len: torch.Tensor
     row_ctx: torch.Tensor
@@ -77,10 +79,12 @@ class HybridCacheManager:
         self._pages: Dict[object, List[int]] = {}
         self._slot: Dict[object, int] = {}
         self._len: Dict[object, int] = {}
+        self._tail: Dict[object, int] = {}       # the last token of each sequence, as of the last advance()
+        self._tail_next: Dict[object, int] = {}  # ... as it will be once the planned step has been advanced
         self.max_seq_pages = (max_tokens + page_size - 1) // page_size
         self.max_rows, self.max_step_tokens = max_rows, max_step_tokens
         self._on_gpu = torch.cuda.is_available() and str(device).startswith("cuda")
-        words = 3 * max_step_tokens + max_rows * (6 + self.max_seq_pages) + \
+        words = 4 * max_step_tokens + max_rows * (6 + self.max_seq_pages) + \
             2 * (max_step_tokens // SCAN_CHUNK + max_rows)
         self._ring = 4 if self._on_gpu else 1
         # a ring of pinned staging buffers (the host may run ahead of the copies), ONE device buffer: the
@@ -132,6 +136,8 @@ class HybridCacheManager:
     def advance(self, rows: Seq[Tuple[object, int]]):
         for sid, n in rows:
             self._len[sid] += n
+            if sid in self._tail_next:
+                self._tail[sid] = self._tail_next.pop(sid)
 
     def free(self, seq_id):
         pages = self._pages.pop(seq_id, None)
@@ -141,6 +147,8 @@ class HybridCacheManager:
         if slot is not None:
             self._free_slots.append(slot)
         self._len.pop(seq_id, None)
+        self._tail.pop(seq_id, None)
+        self._tail_next.pop(seq_id, None)
 
     def reset(self):
         for sid in list(self._slot):
@@ -170,8 +178,8 @@ class HybridCacheManager:
             self._events[i].synchronize()
         host = self._host[i].numpy()
         W = self.max_seq_pages
-        o_ids, o_row, o_pos = 0, T, 2 * T
-        o_rows = 3 * T
+        o_ids, o_row, o_pos, o_prev = 0, T, 2 * T, 3 * T
+        o_rows = 4 * T
         o_bt = o_rows + 4 * B
         start = 0
         max_slot = max_page = 0
@@ -182,6 +190,9 @@ class HybridCacheManager:
             host[o_ids + start:o_ids + start + n] = toks
             host[o_row + start:o_row + start + n] = b
             host[o_pos + start:o_pos + start + n] = range(ctx, ctx + n)
+            host[o_prev + start] = self._tail[sid] if ctx else -1
+            host[o_prev + start + 1:o_prev + start + n] = toks[:-1]
+            self._tail_next[sid] = int(toks[-1])
             host[o_rows + b], host[o_rows + B + b] = start, n
             host[o_rows + 2 * B + b], host[o_rows + 3 * B + b] = ctx, slot
             host[o_bt + b * W:o_bt + b * W + len(pages)] = pages
@@ -214,7 +225,7 @@ class HybridCacheManager:
             self._events[i] = ev
         return RaggedStep(
             tokens=T, rows=B, page=self.page_size, ids=dev[o_ids:o_ids + T], tok_row=dev[o_row:o_row + T],
-            tok_pos=dev[o_pos:o_pos + T], row_start=dev[o_rows:o_rows + B], row_len=dev[o_rows + B:o_rows + 2 * B],
+            tok_pos=dev[o_pos:o_pos + T], tok_prev=dev[o_prev:o_prev + T], row_start=dev[o_rows:o_rows + B], row_len=dev[o_rows + B:o_rows + 2 * B],
             row_ctx=dev[o_rows + 2 * B:o_rows + 3 * B], row_slot=dev[o_rows + 3 * B:o_rows + 4 * B],
             block_table=dev[o_bt:o_bt + B * W].view(B, W), max_slot=max_slot, max_page=max_page, n_chunks=NC,
             ch_start=dev[o_cs:o_cs + NC], ch_len=dev[o_cl:o_cl + NC], row_ch0=dev[o_c0:o_c0 + B],

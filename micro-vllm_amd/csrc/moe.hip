@@ -4,12 +4,17 @@
 //   moe_route    logits = W_router h in fp32 (h in the activation type), the `top` largest (ties: the lower
 //                index), weights = softmax over the chosen logits; beside it sigmoid(w_sg . h), the factor
 //                of a shared expert (one number per token)
+//   moe_route_scored  scores = softmax of the fp32 logits over ALL router outputs; the `top` largest of
+//                score + correction are chosen (ties: the lower index), their weights are the scores themselves
+//                (without the correction) divided by their sum (+ floor), times `scale`.  Router outputs from
+//                `first_pass` on have no expert behind them: they stand for the input itself (moe_combine)
 //   moe_plan     the step's T * top (token, choice) pairs sorted by expert: seg[e] .. seg[e+1] are expert e's
 //                rows, order[i] the pair (token * top + choice) in row i, place[pair] its row.  The order inside
 //                an expert is whatever the atomics give; no result depends on it, since a row's products do
 //                not depend on the other rows (mv_linear_segments)
 //   moe_combine  y_t = sum_k weight[t,k] * expert_out[place[t,k]] (+ factor_t * shared_out_t); with a norm given
-//                the sum goes through it straight into the stream: y += tanh(alpha sum) w + b
+//                the sum goes through it straight into the stream: y += tanh(alpha sum) w + b.  A choice
+//                ids[t,k] >= first_pass adds weight * pass[t] (the feed-forward's own input) instead of an expert's row
 // The experts' products themselves are mv_linear_segments (linear_any.hip) with a SiLU-gate between them.
 #include "common.h"
 
@@ -71,6 +76,61 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const void* h_, int64_t 
     }
 }
 
+template <bool F32>
+__global__ __launch_bounds__(256) void moe_route_scored_kernel(const void* h_, int64_t ldh, const float* wr,
+                                                               const float* correction, int* ids, float* wts, int n,
+                                                               int E, int top, float scale, float floor_) {
+    __shared__ float z[kMaxExperts];
+    const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int e = wv; e < E; e += 4) {
+        const float* w = wr + (int64_t)e * n;
+        float dot = 0.f;
+        if (F32) {
+            const float* h = (const float*)h_ + (int64_t)t * ldh;
+#pragma unroll 8
+            for (int c = lane; c < n; c += 64) dot = fmaf(h[c], w[c], dot);
+        } else {
+            const uint16_t* h = (const uint16_t*)h_ + (int64_t)t * ldh;
+#pragma unroll 8
+            for (int c = lane; c < n; c += 64) dot = fmaf(bf16_bits_to_f32(h[c]), w[c], dot);
+        }
+        dot = wave_sum(dot);
+        if (lane == 0) z[e] = dot;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float largest = z[0], sum = 0.f;
+        for (int e = 1; e < E; ++e) largest = fmaxf(largest, z[e]);
+        for (int e = 0; e < E; ++e) {
+            z[e] = expf(z[e] - largest);
+            sum += z[e];
+        }
+        for (int e = 0; e < E; ++e) z[e] = z[e] / sum;
+        int pick[kMaxTop];
+        float total = 0.f;
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            float bv = -INFINITY;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int j = 0; j < k; ++j) taken |= pick[j] == e;
+                const float c = correction ? z[e] + correction[e] : z[e];
+                if (!taken && (best < 0 || c > bv)) {
+                    best = e;
+                    bv = c;
+                }
+            }
+            pick[k] = best;
+            total += z[best];
+        }
+        total += floor_;
+        for (int k = 0; k < top; ++k) {
+            ids[(int64_t)t * top + k] = pick[k];
+            wts[(int64_t)t * top + k] = (z[pick[k]] / total) * scale;
+        }
+    }
+}
+
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* ids, int* seg, int* order, int* place, int pairs,
                                                         int E) {
     __shared__ int cnt[kMaxExperts + 1];
@@ -104,19 +164,28 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64
                                                           const float* wts, const float* so, int64_t lds_,
                                                           const float* shared_gate, float* y, int64_t ldy, int n,
                                                           int top, const float* norm_w, const float* norm_b,
-                                                          const float* norm_alpha, void* h_, int64_t ldh) {
+                                                          const float* norm_alpha, void* h_, int64_t ldh,
+                                                          const int* ids, int first_pass, const void* pass_,
+                                                          int64_t ldp) {
     const int t = blockIdx.x;
     int rows[kMaxTop];
     float w[kMaxTop];
     for (int k = 0; k < top; ++k) {
         rows[k] = place[(int64_t)t * top + k];
         w[k] = wts[(int64_t)t * top + k];
+        if (ids && ids[(int64_t)t * top + k] >= first_pass) rows[k] = -1;   // the input itself, not an expert's row
     }
     const float g = so ? shared_gate[t] : 0.f;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c < n) {
         float acc = 0.f;
-        for (int k = 0; k < top; ++k) acc = fmaf(w[k], eo[(int64_t)rows[k] * lde + c], acc);
+        for (int k = 0; k < top; ++k) {
+            float v;
+            if (rows[k] >= 0) v = eo[(int64_t)rows[k] * lde + c];
+            else if (F32) v = ((const float*)pass_)[(int64_t)t * ldp + c];
+            else v = bf16_bits_to_f32(((const uint16_t*)pass_)[(int64_t)t * ldp + c]);
+            acc = fmaf(w[k], v, acc);
+        }
         if (so) acc = fmaf(g, so[(int64_t)t * lds_ + c], acc);
         if (norm_w) {
             acc = y[(int64_t)t * ldy + c] + fmaf(tanhf(norm_alpha[0] * acc), norm_w[c], norm_b[c]);
@@ -147,6 +216,20 @@ int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float*
     return check_launch();
 }
 
+int mv_moe_route_scored(const void* h, int64_t ldh, const float* w_router, const float* correction, int32_t* ids,
+                        float* weights, int tokens, int n, int experts, int top, float scale, float sum_floor, int f32,
+                        mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0 || experts <= 0 || experts > kMaxExperts || top <= 0 || top > kMaxTop || top > experts)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!h || !w_router || !ids || !weights || ldh < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(moe_route_scored_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, correction, ids, weights, n, experts, top, scale, sum_floor);
+    else hipLaunchKernelGGL(moe_route_scored_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, correction, ids, weights, n, experts, top, scale, sum_floor);
+    return check_launch();
+}
+
 int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place, int pairs, int experts,
                 mv_stream_t stream) {
     using namespace mv;
@@ -160,7 +243,8 @@ int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place
 int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
                    const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy,
                    const float* norm_w, const float* norm_b, const float* norm_alpha, void* h, int64_t ldh, int tokens,
-                   int n, int top, int f32, mv_stream_t stream) {
+                   int n, int top, int f32, const int32_t* ids, int first_pass, const void* pass, int64_t ldp,
+                   mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || n <= 0 || top <= 0 || top > kMaxTop) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
@@ -168,9 +252,10 @@ int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, c
         (shared_out && lds < n))
         return MV_ERR_INVALID_ARG;
     if (norm_w ? (!norm_b || !norm_alpha || (h && ldh < n)) : h != nullptr) return MV_ERR_INVALID_ARG;
+    if (ids && (!pass || ldp < n || first_pass < 0)) return MV_ERR_INVALID_ARG;
     const dim3 grid(tokens, (n + 255) / 256);
-    if (f32) hipLaunchKernelGGL(moe_combine_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh);
-    else hipLaunchKernelGGL(moe_combine_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh);
+    if (f32) hipLaunchKernelGGL(moe_combine_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh, ids, first_pass, pass, ldp);
+    else hipLaunchKernelGGL(moe_combine_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh, ids, first_pass, pass, ldp);
     return check_launch();
 }
 

@@ -14,8 +14,12 @@
 //   rotary_pairs                   rotate-half rotation of the first `rot` dimensions of each head
 //   gated_group_norm               unit-RMS per group with a SiLU gate before or after it
 //   qk_unitnorm_store              per-head unit-RMS of queries and keys, keys/values into their pages
-//   window_attn                    softmax attention over the last `window` positions with a per-head
-//                                  linear distance penalty
+//   qk_rotary_store                biases on queries and keys, rotation of both over the first `rot` dimensions
+//                                  of a head (adjacent pairs or halves); the rotated key into the key page and the
+//                                  key as projected into the value page (attention whose values are its keys)
+//   window_attn                    softmax attention over the last `window` positions (and, where asked for, the
+//                                  sequence's first `keep_first` positions) with a per-head linear distance
+//                                  penalty and / or a per-head sink in the denominator
 // All of it in fp32; the activation type (bf16 or fp32) only concerns what goes to a projection or
 // into the key/value pages.
 #include "common.h"
@@ -606,18 +610,77 @@ __global__ __launch_bounds__(256) void qk_unitnorm_store_kernel(float* qkv, int6
     }
 }
 
+// One wave per (token, query or key head).  q [T, ld]: heads * d query values then kv_heads * d key values, as
+// one projection leaves them.  The query gets its bias and rotation in place; the key goes, with its bias, unrotated
+// into the value page and rotated into the key page.  angle = position * inv_freq[i], formed in fp64.
+template <bool F32>
+__global__ __launch_bounds__(256) void qk_rotary_store_kernel(float* qk, int64_t ld, const float* qb, const float* kb,
+                                                              void* kc_, void* vc_, const double* inv_freq,
+                                                              PagedRows pr, int T, int H, int G, int d, int rot,
+                                                              int adjacent) {
+    typedef typename ActS<F32>::T T_;
+    T_* kc = (T_*)kc_;
+    T_* vc = (T_*)vc_;
+    const int per = H + G;
+    const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (unit >= (int64_t)T * per) return;
+    const int t = (int)(unit / per), u = (int)(unit % per);
+    const int pos = pr.tok_pos[t];
+    float* p = qk + (int64_t)t * ld + (int64_t)u * d;
+    const float* bias = u < H ? (qb ? qb + (int64_t)u * d : nullptr) : (kb ? kb + (int64_t)(u - H) * d : nullptr);
+    T_* kdst = nullptr;
+    T_* vdst = nullptr;
+    if (u >= H) {
+        const int pg = pr.block_table[(int64_t)pr.tok_row[t] * pr.bt_stride + pos / pr.page];
+        if (pg < 0) return;
+        const int64_t slot = ((int64_t)pg * pr.page + pos % pr.page) * G + (u - H);
+        kdst = kc + slot * d;
+        vdst = vc + slot * d;
+    }
+    const int half = rot / 2;
+    for (int i = lane; i < half; i += 64) {
+        const int a = adjacent ? 2 * i : i, b = adjacent ? 2 * i + 1 : i + half;
+        const double ang = (double)pos * inv_freq[i];
+        const float cs = (float)cos(ang), sn = (float)sin(ang);
+        const float x0 = bias ? p[a] + bias[a] : p[a], x1 = bias ? p[b] + bias[b] : p[b];
+        const float r0 = x0 * cs - x1 * sn, r1 = x1 * cs + x0 * sn;
+        if (u < H) {
+            p[a] = r0;
+            p[b] = r1;
+        } else {
+            ActS<F32>::st(kdst + a, r0);
+            ActS<F32>::st(kdst + b, r1);
+            ActS<F32>::st(vdst + a, x0);
+            ActS<F32>::st(vdst + b, x1);
+        }
+    }
+    for (int c = rot + lane; c < d; c += 64) {
+        const float x0 = bias ? p[c] + bias[c] : p[c];
+        if (u < H) {
+            p[c] = x0;
+        } else {
+            ActS<F32>::st(kdst + c, x0);
+            ActS<F32>::st(vdst + c, x0);
+        }
+    }
+}
+
 constexpr int kMaxVC = 4;  // value columns per lane: vdim <= 256
 
 // One workgroup per (token, head).  Its NW waves (4, or 16 when a step has too few tokens to fill the
 // chip otherwise: decoding) take the window's 64-key tiles in turn: a lane scores
 // one key (q from LDS, the key row straight from its page), the wave forms max / sum of the tile and
 // then, lanes now owning value columns, adds the tile's weighted values; the waves' partial softmaxes
-// meet in LDS.  The same code serves a prompt's portion and a single decoded token.
+// meet in LDS.  The same code serves a prompt's portion and a single decoded token.  Positions below
+// `keep_first` stay visible after the window has passed them (a second run of tiles, at their true
+// positions); sinks[h] joins the denominator as exp(sink) with no key and no value.
 template <bool F32, int NW>
 __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
                                                           const void* vc_, void* out_, int64_t ldo, PagedRows pr,
                                                           const float* slopes, int T, int H, int G, int d, int dv,
-                                                          float scale, int window, const int* row_len, int max_len) {
+                                                          float scale, int window, const int* row_len, int max_len,
+                                                          int keep_first, const float* sinks) {
     typedef typename ActS<F32>::T T_;
     extern __shared__ float lds[];
     if (max_len > 0 && row_len[pr.tok_row[blockIdx.x / H]] > max_len) return;   // the tiled kernel's rows
@@ -638,10 +701,13 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
     for (int c = threadIdx.x; c < d; c += 64 * NW) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
     __syncthreads();
     float m = -INFINITY, l = 0.f, acc[kMaxVC] = {0.f, 0.f, 0.f, 0.f};
-    for (int j0 = lo + 64 * wv; j0 <= pos; j0 += 64 * NW) {
+    const int kept = keep_first < lo ? keep_first : lo;    // kept positions the window no longer covers: [0, kept)
+    for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+    const int first = run ? lo : 0, last = run ? pos : kept - 1;
+    for (int j0 = first + 64 * wv; j0 <= last; j0 += 64 * NW) {
         const int j = j0 + lane;
         float s = -INFINITY;
-        if (j <= pos) {
+        if (j <= last) {
             const int pg = bt[j / pr.page];
             const T_* kr = kc + (((int64_t)pg * pr.page + j % pr.page) * G + g) * d;
             float dot = 0.f;
@@ -661,14 +727,14 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
             s = dot * scale - slope * (float)(pos - j);
         }
         const float mn = fmaxf(m, wave_max(s));
-        const float pj_ = j <= pos ? expf(s - mn) : 0.f;
+        const float pj_ = j <= last ? expf(s - mn) : 0.f;
         const float corr = expf(m - mn);   // m = -inf on the wave's first tile: exp(-inf) = 0
         l = l * corr + wave_sum(pj_);
         m = mn;
         __builtin_amdgcn_wave_barrier();
         ps[lane] = pj_;
         __builtin_amdgcn_wave_barrier();
-        const int cnt = pos - j0 + 1 < 64 ? pos - j0 + 1 : 64;
+        const int cnt = last - j0 + 1 < 64 ? last - j0 + 1 : 64;
 #pragma unroll
         for (int ci = 0; ci < kMaxVC; ++ci) acc[ci] *= corr;
         // eight value rows at a time, their loads in flight together (a tile of 64 keys lies in two pages at
@@ -700,6 +766,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
             }
         }
     }
+    }
     if (lane == 0) {
         mm[wv] = m;
         ll[wv] = l;
@@ -714,7 +781,12 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
         float M = mm[0];                                   // wave 0 always has a key: finite
 #pragma unroll
         for (int w = 1; w < NW; ++w) M = fmaxf(M, mm[w]);
-        float w4[NW], L = 0.f;
+        float L = 0.f;
+        if (sinks) {
+            M = fmaxf(M, sinks[h]);
+            L = expf(sinks[h] - M);
+        }
+        float w4[NW];
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             w4[w] = expf(mm[w] - M);   // a wave without keys: exp(-inf) = 0
@@ -746,7 +818,7 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
                                                                const uint16_t* vc, uint16_t* out, int64_t ldo,
                                                                PagedRows pr, const int* ch_start, const int* ch_len,
                                                                const float* slopes, int H, int G, float scale,
-                                                               int window) {
+                                                               int window, int keep_first, const float* sinks) {
     constexpr int D = KS * 32, DV = CT * 16, SK = D + 8, SV = DV + 8;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[64][SK];
     __shared__ __attribute__((aligned(16))) uint16_t Vs[64][SV];
@@ -777,7 +849,10 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
     const float slope = slopes ? slopes[h] : 0.f;
     const int klo = p0 - window + 1 > 0 ? p0 - window + 1 : 0, khi = p0 + len - 1;
     const int wq_lo = p0 + 16 * wv, wq_hi = wq_lo + 15;   // this wave's query positions
-    for (int kt = klo / 64; kt <= khi / 64; ++kt) {
+    // key tiles: those of the kept first positions that the window of the chunk's first query has left behind,
+    // then the window's
+    const int kt_lo = klo / 64, kt_keep = ((keep_first < klo ? keep_first : klo) + 63) / 64;
+    for (int kt = kt_keep > 0 ? 0 : kt_lo; kt <= khi / 64; kt = (kt + 1 >= kt_keep && kt + 1 < kt_lo) ? kt_lo : kt + 1) {
         const int kbase = kt * 64;
         const int64_t pgrow = (int64_t)bt[kt] * 64;
         __syncthreads();
@@ -790,7 +865,8 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
             st16(&Vs[rr][cc * 8], ld16(vc + ((pgrow + rr) * G + g) * DV + cc * 8));
         }
         __syncthreads();
-        if (kbase > wq_hi || kbase + 63 <= wq_lo - window) continue;   // nothing of this tile is visible to the wave
+        // nothing of this tile is visible to the wave
+        if (kbase > wq_hi || (kbase + 63 <= wq_lo - window && kbase >= keep_first)) continue;
         f32x4_t sc[4];
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) {
@@ -807,7 +883,7 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int kpos = kbase + 16 * nt + 4 * qd + j;
-                const bool ok = qok && kpos <= qpos && kpos > qpos - window;
+                const bool ok = qok && kpos <= qpos && (kpos > qpos - window || kpos < keep_first);
                 const float v = ok ? sc[nt][j] * scale - slope * (float)(qpos - kpos) : -INFINITY;
                 sc[nt][j] = v;
                 mx = fmaxf(mx, v);
@@ -842,7 +918,11 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
             }
     }
     if (qok) {
-        const float inv = 1.0f / l;
+        float inv = 1.0f / l;
+        if (sinks) {   // one more term of the denominator, without a value (m is finite: a query sees itself)
+            const float sk = sinks[h], mn = fmaxf(m, sk);
+            inv = expf(m - mn) / (l * expf(m - mn) + expf(sk - mn));
+        }
         uint16_t* op = out + (int64_t)(start + myq) * ldo + (int64_t)h * DV + 4 * qd;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -1107,14 +1187,34 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
     return check_launch();
 }
 
+int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* k_bias, void* k_cache, void* v_cache,
+                       const double* inv_freq, const int32_t* tok_row, const int32_t* tok_pos,
+                       const int32_t* block_table, int bt_stride, int page, int tokens, int heads, int kv_heads, int d,
+                       int rot, int adjacent, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || page <= 0 || rot < 0 || rot > d || rot % 2)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!qk || !k_cache || !v_cache || (rot > 0 && !inv_freq) || !tok_row || !tok_pos || !block_table ||
+        ld < (int64_t)(heads + kv_heads) * d)
+        return MV_ERR_INVALID_ARG;
+    PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
+    const int64_t units = (int64_t)tokens * (heads + kv_heads);
+    const dim3 grid((unsigned)((units + 3) / 4));
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(qk_rotary_store_kernel<true>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent);
+    else hipLaunchKernelGGL(qk_rotary_store_kernel<false>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent);
+    return check_launch();
+}
+
 int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
-                   int chunks, int max_len, mv_stream_t stream) {
+                   int chunks, int max_len, int keep_first, const float* sinks, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || window <= 0 ||
-        heads % kv_heads)
+        heads % kv_heads || keep_first < 0)
         return MV_ERR_INVALID_ARG;
     if (dv > 64 * kMaxVC || d > 4096) return MV_ERR_UNSUPPORTED;
     if (tokens == 0) return MV_OK;
@@ -1133,7 +1233,7 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
 #define MV_WA_TILE(KS_, CT_)                                                                                         \
     hipLaunchKernelGGL((window_attn_tile_kernel<KS_, CT_>), tg, dim3(256), 0, s, q, ldq, (const uint16_t*)k_cache,      \
                        (const uint16_t*)v_cache, (uint16_t*)out, ldo, pr, ch_start, ch_len, slopes, heads, kv_heads, scale, \
-                       window);                                                                                       \
+                       window, keep_first, sinks);                                                                                    \
     skip_len = max_len
         if (d == 64 && dv == 64) { MV_WA_TILE(2, 4); }
         else if (d == 96 && dv == 96) { MV_WA_TILE(3, 6); }
@@ -1149,11 +1249,11 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
     const size_t lds = (size_t)(d + 64 * nw + 2 * nw + nw * dv) * sizeof(float);
     if (lds > 64 * 1024) return MV_ERR_UNSUPPORTED;
     if (wide) {
-        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
-        else hipLaunchKernelGGL((window_attn_kernel<false, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len, keep_first, sinks);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len, keep_first, sinks);
     } else {
-        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
-        else hipLaunchKernelGGL((window_attn_kernel<false, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len, keep_first, sinks);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len, keep_first, sinks);
     }
     return check_launch();
 }

@@ -18,6 +18,13 @@
 //   gelu_gate_rows:      out = act( gelu_tanh(a) * table[id][off .. off+n) )
 //   silu_mul:            out = act( silu(a[:, :n]) * a[:, n:2n] )
 //   sigmoid_gate:        out = act( a * sigmoid(g) )   (g == NULL: act(a))
+//   embed_pair:          x = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets]   (a hashed
+//                        table over pairs of neighbouring tokens; row `buckets` where a token has no predecessor)
+//   add_rmsnorm:         x += y1 (+ y2); h = act( x / sqrt(mean(x^2) + eps) * w )   (the sublayers of a parallel
+//                        layer enter the stream together and the next layer's norm comes out of the same launch)
+//   rmsnorm_gather:      out = act( x[idx] / sqrt(mean(x[idx]^2) + eps) * (offset + w) )
+//   gated_act:           out = act( f(a[:, :n]) * a[:, n:2n] ), f = SiLU or the tanh form of GELU; or the clamped
+//                        gate  g' = min(g, limit), u' = clamp(u, +-limit): out = act( g' sigmoid(slope g') (u' + 1) )
 // All arithmetic is fp32 with the library's exact division, square root and tanh.
 #include "common.h"
 
@@ -79,8 +86,8 @@ __global__ __launch_bounds__(256) void postnorm_residual_kernel(const float* y1,
 
 template <bool F32>
 __global__ __launch_bounds__(256) void offset_rmsnorm_gather_kernel(const float* x, int64_t ldx, const int* idx,
-                                                                    const float* w, float eps, void* out_,
-                                                                    int64_t ldo, int n) {
+                                                                    const float* w, float eps, float offset,
+                                                                    void* out_, int64_t ldo, int n) {
     typedef typename Act<F32>::T T;
     __shared__ float red[4];
     T* out = (T*)out_;
@@ -90,7 +97,7 @@ __global__ __launch_bounds__(256) void offset_rmsnorm_gather_kernel(const float*
     for (int c = threadIdx.x; c < n; c += 256) ss += a[c] * a[c];
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)n + eps);
-    for (int c = threadIdx.x; c < n; c += 256) Act<F32>::st(out + (int64_t)row * ldo + c, (a[c] * inv) * (1.0f + w[c]));
+    for (int c = threadIdx.x; c < n; c += 256) Act<F32>::st(out + (int64_t)row * ldo + c, (a[c] * inv) * (offset + w[c]));
 }
 
 template <bool F32>
@@ -261,6 +268,74 @@ __global__ __launch_bounds__(256) void sigmoid_gate_kernel(const float* a, int64
     Act<F32>::st(out + row * ldo + c, v);
 }
 
+// ---- pair-hashed embedding, parallel layers behind one norm, gated activations ----------------------------
+template <bool F32>
+__global__ __launch_bounds__(256) void embed_pair_kernel(const void* table_, const void* pairs_, const int* ids,
+                                                         const int* prev, float* x, int64_t ldx, int n, int vocab,
+                                                         int64_t buckets, int64_t mul_prev, int64_t mul_cur,
+                                                         float scale) {
+    typedef typename Act<F32>::T T;
+    const T* table = (const T*)table_;
+    const T* pairs = (const T*)pairs_;
+    const int row = blockIdx.x;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const int pv = prev[row];
+    // every factor reduced first: the products stay below 2^62 for any 31-bit bucket count
+    const int64_t r = pv < 0 ? buckets
+                             : (((int64_t)pv % buckets) * (mul_prev % buckets) % buckets +
+                                ((int64_t)id % buckets) * (mul_cur % buckets) % buckets) % buckets;
+    for (int c = threadIdx.x; c < n; c += 256)
+        x[(int64_t)row * ldx + c] = Act<F32>::ld(table + (int64_t)id * n + c) * scale + Act<F32>::ld(pairs + r * n + c);
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float* y1, int64_t ld1, const float* y2, int64_t ld2,
+                                                          float* x, int64_t ldx, const float* w, float eps, void* h_,
+                                                          int64_t ldh, int n) {
+    typedef typename Act<F32>::T T;
+    __shared__ float red[4];
+    T* h = (T*)h_;
+    const int row = blockIdx.x;
+    float* xr = x + (int64_t)row * ldx;
+    float ss = 0.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < n; c += 256) {
+        float v = xr[c];
+        if (y1) {
+            v += y2 ? y1[(int64_t)row * ld1 + c] + y2[(int64_t)row * ld2 + c] : y1[(int64_t)row * ld1 + c];
+            xr[c] = v;
+        }
+        ss += v * v;
+    }
+    if (!w) return;
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll 4
+    for (int c = threadIdx.x; c < n; c += 256) Act<F32>::st(h + (int64_t)row * ldh + c, (xr[c] * inv) * w[c]);
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void gated_act_kernel(const float* a, int64_t lda, void* out_, int64_t ldo, int n,
+                                                        int kind, float limit, float slope) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= n) return;
+    float g = a[row * lda + c], u = a[row * lda + n + c], v;
+    if (kind == 0) {
+        v = (g / (1.0f + expf(-g))) * u;
+    } else if (kind == 1) {
+        v = gelu_tanh_f(g) * u;
+    } else {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        v = (g / (1.0f + expf(-slope * g))) * (u + 1.0f);
+    }
+    Act<F32>::st(out + row * ldo + c, v);
+}
+
 }  // namespace mv
 
 extern "C" {
@@ -292,13 +367,58 @@ int mv_postnorm_residual(const float* y1, int64_t ld1, const float* y2, int64_t 
 
 int mv_offset_rmsnorm_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, float eps, void* out,
                              int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
+    return mv_rmsnorm_gather(x, ldx, idx, w, eps, 1.0f, out, ldo, rows, n, f32, stream);
+}
+
+int mv_rmsnorm_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, float eps, float offset,
+                      void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
     using namespace mv;
     if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
     if (rows == 0) return MV_OK;
     if (!x || !w || !out || ldx < n || ldo < n) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(offset_rmsnorm_gather_kernel<true>, dim3(rows), dim3(256), 0, s, x, ldx, idx, w, eps, out, ldo, n);
-    else hipLaunchKernelGGL(offset_rmsnorm_gather_kernel<false>, dim3(rows), dim3(256), 0, s, x, ldx, idx, w, eps, out, ldo, n);
+    if (f32) hipLaunchKernelGGL(offset_rmsnorm_gather_kernel<true>, dim3(rows), dim3(256), 0, s, x, ldx, idx, w, eps, offset, out, ldo, n);
+    else hipLaunchKernelGGL(offset_rmsnorm_gather_kernel<false>, dim3(rows), dim3(256), 0, s, x, ldx, idx, w, eps, offset, out, ldo, n);
+    return check_launch();
+}
+
+int mv_embed_pair(const void* table, const void* pairs, const int32_t* ids, const int32_t* prev, float* x, int64_t ldx,
+                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale, int f32,
+                  mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || vocab <= 0 || buckets <= 0 || buckets > 0x7fffffff || mul_prev < 0 || mul_cur < 0)
+        return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!table || !pairs || !ids || !prev || !x || ldx < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(embed_pair_kernel<true>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale);
+    else hipLaunchKernelGGL(embed_pair_kernel<false>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale);
+    return check_launch();
+}
+
+int mv_add_rmsnorm(const float* y1, int64_t ld1, const float* y2, int64_t ld2, float* x, int64_t ldx, const float* w,
+                   float eps, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!x || ldx < n || (y1 && ld1 < n) || (y2 && (!y1 || ld2 < n)) || (w && (!h || ldh < n)) || (!w && !y1))
+        return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(add_rmsnorm_kernel<true>, dim3(rows), dim3(256), 0, s, y1, ld1, y2, ld2, x, ldx, w, eps, h, ldh, n);
+    else hipLaunchKernelGGL(add_rmsnorm_kernel<false>, dim3(rows), dim3(256), 0, s, y1, ld1, y2, ld2, x, ldx, w, eps, h, ldh, n);
+    return check_launch();
+}
+
+int mv_gated_act(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int kind, float limit,
+                 float slope, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || kind < 0 || kind > 2) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !out || lda < 2 * (int64_t)n || ldo < n) return MV_ERR_INVALID_ARG;
+    const dim3 grid(rows, (n + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(gated_act_kernel<true>, grid, dim3(256), 0, s, a, lda, out, ldo, n, kind, limit, slope);
+    else hipLaunchKernelGGL(gated_act_kernel<false>, grid, dim3(256), 0, s, a, lda, out, ldo, n, kind, limit, slope);
     return check_launch();
 }
 

@@ -220,10 +220,34 @@ def qk_unitnorm_store(qkv, k_cache, v_cache, step, heads: int, kv_heads: int, d:
         kv_heads, d, dv, float(eps), _is_f32(k_cache), nv.stream_ptr()))
 
 
+def qk_rotary_store(qk, q_bias, k_bias, k_cache, v_cache, inv_freq, step, heads: int, kv_heads: int, d: int, rot: int,
+                    adjacent: bool = True):
+    """qk [T, (heads + kv_heads) * d] fp32 = queries then keys of one projection.  Biases are added, queries rotated
+    in place; a key goes rotated into k_cache and as projected (with its bias) into v_cache: the values of this
+    attention are its unrotated keys."""
+    tokens = qk.shape[0]
+    assert qk.shape[1] == (heads + kv_heads) * d and step.tokens == tokens
+    page = k_cache.shape[1]
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype
+    assert k_cache.shape[1:] == (page, kv_heads, d) and v_cache.shape == k_cache.shape
+    assert int(step.max_page) < k_cache.shape[0] and page == step.page
+    assert q_bias is None or (q_bias.numel() == heads * d and q_bias.is_contiguous())
+    assert k_bias is None or (k_bias.numel() == kv_heads * d and k_bias.is_contiguous())
+    assert rot == 0 or (inv_freq.is_cuda and inv_freq.dtype == torch.float64 and inv_freq.numel() == rot // 2)
+    nv.check("mv_qk_rotary_store", nv.lib().mv_qk_rotary_store(
+        _f32(qk).data_ptr(), _ld(qk), None if q_bias is None else _f32(q_bias).data_ptr(),
+        None if k_bias is None else _f32(k_bias).data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        None if rot == 0 else inv_freq.data_ptr(), step.tok_row.data_ptr(), step.tok_pos.data_ptr(),
+        step.block_table.data_ptr(), step.block_table.stride(0), page, tokens, heads, kv_heads, d, rot, int(adjacent),
+        _is_f32(k_cache), nv.stream_ptr()))
+
+
 def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: int, d: int, dv: int,
-                scale: float, window: int, tiled: bool = True):
+                scale: float, window: int, tiled: bool = True, keep_first: int = 0, sinks=None):
     """`tiled`: rows of more than SCAN_SEQ_MAX tokens go to the matrix-core kernel where it applies (bf16,
-    the head shapes it is built for); False keeps every token on the plain kernel."""
+    the head shapes it is built for); False keeps every token on the plain kernel.  `keep_first`: positions below it
+    stay visible behind the window; `sinks` [heads]: exp(sink) joins each head's denominator."""
+    assert sinks is None or (sinks.numel() == heads and sinks.is_contiguous())
     tokens = q.shape[0]
     assert q.shape[1] >= heads * d and out.shape == (tokens, heads * dv) and out.dtype == k_cache.dtype
     page = k_cache.shape[1]
@@ -236,7 +260,8 @@ def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: in
         page, None if slopes is None else _f32(slopes).data_ptr(), tokens, heads, kv_heads, d, dv, float(scale),
         int(window), _is_f32(k_cache), step.row_len.data_ptr(),
         step.ch_start.data_ptr() if step.n_chunks else None, step.ch_len.data_ptr() if step.n_chunks else None,
-        step.n_chunks if tiled else 0, SCAN_SEQ_MAX, nv.stream_ptr()))
+        step.n_chunks if tiled else 0, SCAN_SEQ_MAX, int(keep_first), None if sinks is None else _f32(sinks).data_ptr(),
+        nv.stream_ptr()))
 
 
 # ---------------------------------------------------------------------------------------------------------
@@ -452,12 +477,16 @@ def moe_plan(ids, seg, order, place, experts: int):
         nv.stream_ptr()))
 
 
-def moe_combine(expert_out, place, weights, shared_out, shared_gate, y, norm=None, h=None):
+def moe_combine(expert_out, place, weights, shared_out, shared_gate, y, norm=None, h=None, ids=None, first_pass: int = 0,
+                passed=None):
     """y = the weighted sum of each token's experts (+ shared_gate * shared_out).  With `norm` y is the residual
     stream and receives the sum through that norm, y += tanh(alpha sum) w + b; h (optional) = y in the activation
-    type."""
+    type.  With `ids` [tokens, top] a choice >= first_pass is an expert that hands its input through: it adds its
+    weight times the token's row of `passed` (activation type)."""
     tokens, n = y.shape
     top = weights.shape[1]
+    assert ids is None or (ids.numel() == tokens * top and passed is not None and passed.shape == (tokens, n)
+                           and passed.stride(1) == 1)
     assert expert_out.shape == (tokens * top, n) and place.numel() == tokens * top and weights.is_contiguous()
     assert shared_out is None or (shared_out.shape == (tokens, n) and shared_gate.numel() == tokens)
     assert h is None or (norm is not None and h.shape == (tokens, n))
@@ -467,4 +496,69 @@ def moe_combine(expert_out, place, weights, shared_out, shared_gate, y, norm=Non
         None if shared_out is None else _f32(shared_out).data_ptr(), 0 if shared_out is None else _ld(shared_out),
         None if shared_out is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y), w, b, a,
         None if h is None else h.data_ptr(), 0 if h is None else _ld(h), tokens, n, top,
-        0 if h is None else _is_f32(h), nv.stream_ptr()))
+        _is_f32(passed) if passed is not None else (0 if h is None else _is_f32(h)),
+        None if ids is None else _i32(ids).data_ptr(), int(first_pass), None if ids is None else passed.data_ptr(),
+        0 if ids is None else _ld(passed), nv.stream_ptr()))
+
+
+def moe_route_scored(h, w_router, correction, ids, weights, scale: float, sum_floor: float):
+    """Scores = softmax over all router outputs; the `top` largest of score + correction are chosen, their weights are
+    the scores divided by their sum (+ sum_floor), times scale."""
+    tokens, n = h.shape
+    E, top = w_router.shape[0], ids.shape[1]
+    assert h.stride(1) == 1 and w_router.shape == (E, n) and w_router.is_contiguous()
+    assert ids.shape == (tokens, top) and weights.shape == (tokens, top) and ids.is_contiguous()
+    assert weights.is_contiguous() and ids.dtype == torch.int32
+    assert correction is None or (correction.numel() == E and correction.is_contiguous())
+    nv.check("mv_moe_route_scored", nv.lib().mv_moe_route_scored(
+        h.data_ptr(), _ld(h), _f32(w_router).data_ptr(), None if correction is None else _f32(correction).data_ptr(),
+        ids.data_ptr(), _f32(weights).data_ptr(), tokens, n, E, top, float(scale), float(sum_floor), _is_f32(h),
+        nv.stream_ptr()))
+
+
+GATE_SILU, GATE_GELU_TANH, GATE_CLAMPED = 0, 1, 2
+
+
+def gated_act(a, out, kind: int, limit: float = 0.0, slope: float = 1.0):
+    """out = act(f(a[:, :n]) * a[:, n:]) with f = SiLU / GELU (tanh form), or the clamped gate
+    min(g, limit) * sigmoid(slope * min(g, limit)) * (clamp(u, -limit, limit) + 1)."""
+    rows, n = out.shape
+    assert a.shape == (rows, 2 * n)
+    nv.check("mv_gated_act", nv.lib().mv_gated_act(
+        _f32(a).data_ptr(), _ld(a), out.data_ptr(), _ld(out), rows, n, int(kind), float(limit), float(slope),
+        _is_f32(out), nv.stream_ptr()))
+
+
+def embed_pair(table, pairs, ids, prev, x, scale: float, buckets: int, mul_prev: int, mul_cur: int):
+    """x = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets], row `buckets` where prev < 0."""
+    rows, n = x.shape
+    assert table.is_cuda and table.is_contiguous() and table.shape[1] == n and table.dtype == pairs.dtype
+    assert pairs.is_cuda and pairs.is_contiguous() and pairs.shape == (buckets + 1, n)
+    assert ids.numel() == rows and prev.numel() == rows
+    nv.check("mv_embed_pair", nv.lib().mv_embed_pair(
+        table.data_ptr(), pairs.data_ptr(), _i32(ids).data_ptr(), _i32(prev).data_ptr(), _f32(x).data_ptr(), _ld(x),
+        rows, n, table.shape[0], int(buckets), int(mul_prev), int(mul_cur), float(scale), _is_f32(table),
+        nv.stream_ptr()))
+
+
+def add_rmsnorm(x, y1=None, y2=None, w=None, eps: float = 0.0, h=None):
+    """x += y1 (+ y2); with `w`: h = act(x / sqrt(mean(x^2) + eps) * w)."""
+    rows, n = x.shape
+    assert y1 is None or y1.shape == (rows, n)
+    assert y2 is None or (y1 is not None and y2.shape == (rows, n))
+    assert (w is None) == (h is None) and (w is None or (w.numel() == n and w.is_contiguous() and h.shape == (rows, n)))
+    nv.check("mv_add_rmsnorm", nv.lib().mv_add_rmsnorm(
+        None if y1 is None else _f32(y1).data_ptr(), 0 if y1 is None else _ld(y1),
+        None if y2 is None else _f32(y2).data_ptr(), 0 if y2 is None else _ld(y2), _f32(x).data_ptr(), _ld(x),
+        None if w is None else _f32(w).data_ptr(), float(eps), None if h is None else h.data_ptr(),
+        0 if h is None else _ld(h), rows, n, 0 if h is None else _is_f32(h), nv.stream_ptr()))
+
+
+def rmsnorm_gather(x, idx, w, eps: float, out, offset: float = 0.0):
+    """out = act(x[idx] / sqrt(mean(x[idx]^2) + eps) * (offset + w))."""
+    rows, n = out.shape
+    assert x.shape[1] == n and w.numel() == n and w.is_contiguous()
+    assert idx is None or idx.numel() == rows
+    nv.check("mv_rmsnorm_gather", nv.lib().mv_rmsnorm_gather(
+        _f32(x).data_ptr(), _ld(x), None if idx is None else _i32(idx).data_ptr(), _f32(w).data_ptr(), float(eps),
+        float(offset), out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))

@@ -6,7 +6,7 @@ A family = (configuration reader, model object, runner and cache manager the eng
              ModelGraphRunner / KVCacheManager);
   "ragged" - stacks with an fp32 residual stream whose layers are listed one by one (recurrent
              mixers, windowed or latent attention, dense or routed feed-forwards), run step by step
-             over ragged batches (RaggedRunner / HybridCacheManager): Pagazen, Fagunex.
+             over ragged batches (RaggedRunner / HybridCacheManager): Pagazen, Fagunex, Nesisun.
 """
 from typing import Callable, Dict
 
@@ -36,8 +36,18 @@ def _load_fagunex(config_json, files, name):
     return FagunexModel(cfg, files)
 
 
+def _load_nesisun(config_json, files, name):
+    from .nesisun import NesisunConfig, NesisunModel, tensor_shapes
+    cfg = NesisunConfig.from_json(config_json, name)
+    for tensor, shape in tensor_shapes(cfg).items():
+        if tensor not in files:
+            raise KeyError(f"tensor {tensor!r} {shape} is not in the checkpoint")
+    return NesisunModel(cfg, files)
+
+
 register("Pagazen", _load_pagazen)
 register("Fagunex", _load_fagunex)
+register("Nesisun", _load_nesisun)
 
 
 def loader_for(config_json: dict):
