@@ -79,6 +79,14 @@ def parse():
                          "at equal width and depth; one JSON line of its own")
     ap.add_argument("--fagunex-widths", default="1024,2048,4096")
     ap.add_argument("--fagunex-kernels", action="store_true", help="with --fagunex: per-op times of one step on stderr")
+    ap.add_argument("--nesisun", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the Nesisun design "
+                         "(parallel layers behind one norm, windowed attention with kept first positions and a sink "
+                         "whose values are its keys, dense and routed feed-forwards; random weights) at a few widths, "
+                         "with dense feed-forwards only and with every second one routed, beside the Llama-shaped "
+                         "model of equal width, depth and feed-forward parameters; one JSON line of its own")
+    ap.add_argument("--nesisun-widths", default="1024,2048,4096")
+    ap.add_argument("--nesisun-kernels", action="store_true", help="with --nesisun: per-op times of one step on stderr")
     return ap.parse_args()
 
 
@@ -587,49 +595,60 @@ def pagazen_compare(args, dev):
         del eng
         torch.cuda.empty_cache()
         # ---- Llama-shaped, equal width / depth; gate+up+down hold what up+down of 4 x width hold ----
-        ffn = (8 * width // 3 + 255) // 256 * 256
-        lc = SyntheticConfig(f"llama-w{width}", 32000, width, layers, width // 128, max(1, width // 512), 128, ffn, 1e-5)
-        model = build_synthetic_model(lc, dev, seed=1)
-        blocks = (S + 300) // 256 + 2
-        common = dict(model=model, num_layers=layers, num_heads=lc.num_attention_heads, head_size=128,
-                      kv_num_heads=lc.num_key_value_heads, hidden_dim=width, intermediate_size=lc.intermediate_size,
-                      device=dev, max_blocks=max(32, blocks))
-        pre = ModelPrefillRunner(max_batch_size=1, **common)
-        mgr = KVCacheManager(blocks + 1, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16, device=dev,
-                             max_tokens=blocks * 256, max_batch_size=1)
-        assert mgr.alloc(0, S)[0]
-        mgr.cache_batch_data([0], [S])
-        pids = torch.tensor([ids]).to(dev)
-        ms = _events_ms(lambda: pre.forward(pids, mgr, 1, last_token_only=True), 3)
-        row["llama_prefill_tok_s"] = round(S / ms * 1e3, 1)
-        del pre, mgr
-        for bs in (1, 8):
-            dec = ModelGraphRunner(max_batch_size=bs, **common)
-            mgr = KVCacheManager(bs * blocks + 2, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16,
-                                 device=dev, max_tokens=blocks * 256, max_batch_size=bs)
-            for sid in range(bs):
-                assert mgr.alloc(sid, S)[0]
-            dec.capture(mgr, batch_sizes=[bs])
-            tok = torch.zeros(bs, dtype=torch.long, device=dev)
-            pos = [S + 1]
-
-            def step():
-                for sid in range(bs):
-                    mgr.append(sid)
-                mgr.cache_batch_data(list(range(bs)), [pos[0]] * bs)
-                pos[0] += 1
-                return dec.greedy_ids(dec.forward(tok, mgr, bs))
-            ms = _events_ms(step, 20)
-            row[f"llama_decode_bs{bs}_tok_s"] = round(bs / ms * 1e3, 1)
-            row[f"llama_decode_bs{bs}_ms"] = round(ms, 3)
-            del dec, mgr
-        row["llama_weight_GB"] = round(lc.weight_bytes() / 1e9, 3)
-        del model
-        torch.cuda.empty_cache()
+        row.update(_llama_row(dev, width, layers, S, ids, (8 * width // 3 + 255) // 256 * 256))
         log(f"[bench] {row}")
         rows.append(row)
     print(json.dumps({"metric": "Pagazen beside the Llama-shaped family: prefill and decode tokens/s at equal size",
                       "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
+
+
+def _llama_row(dev, width, layers, S, ids, ffn):
+    """The Llama-shaped runners (padded prefill, graph-captured decode) at the given width / depth / feed-forward
+    width: prefill of one prompt of S tokens, decode at bs 1 / 8 behind it."""
+    from micro_vllm_amd.core.cache_manager import KVCacheManager
+    from micro_vllm_amd.core.layer.model_graph import ModelGraphRunner
+    from micro_vllm_amd.core.layer.model_prefill import ModelPrefillRunner
+    from micro_vllm_amd.models import SyntheticConfig, build_synthetic_model
+    row = {}
+    lc = SyntheticConfig(f"llama-w{width}", 32000, width, layers, width // 128, max(1, width // 512), 128, ffn, 1e-5)
+    model = build_synthetic_model(lc, dev, seed=1)
+    blocks = (S + 300) // 256 + 2
+    common = dict(model=model, num_layers=layers, num_heads=lc.num_attention_heads, head_size=128,
+                  kv_num_heads=lc.num_key_value_heads, hidden_dim=width, intermediate_size=lc.intermediate_size,
+                  device=dev, max_blocks=max(32, blocks))
+    pre = ModelPrefillRunner(max_batch_size=1, **common)
+    mgr = KVCacheManager(blocks + 1, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16, device=dev,
+                         max_tokens=blocks * 256, max_batch_size=1)
+    assert mgr.alloc(0, S)[0]
+    mgr.cache_batch_data([0], [S])
+    pids = torch.tensor([ids]).to(dev)
+    ms = _events_ms(lambda: pre.forward(pids, mgr, 1, last_token_only=True), 3)
+    row["llama_prefill_tok_s"] = round(S / ms * 1e3, 1)
+    del pre, mgr
+    for bs in (1, 8):
+        dec = ModelGraphRunner(max_batch_size=bs, **common)
+        mgr = KVCacheManager(bs * blocks + 2, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16,
+                             device=dev, max_tokens=blocks * 256, max_batch_size=bs)
+        for sid in range(bs):
+            assert mgr.alloc(sid, S)[0]
+        dec.capture(mgr, batch_sizes=[bs])
+        tok = torch.zeros(bs, dtype=torch.long, device=dev)
+        pos = [S + 1]
+
+        def step():
+            for sid in range(bs):
+                mgr.append(sid)
+            mgr.cache_batch_data(list(range(bs)), [pos[0]] * bs)
+            pos[0] += 1
+            return dec.greedy_ids(dec.forward(tok, mgr, bs))
+        ms = _events_ms(step, 20)
+        row[f"llama_decode_bs{bs}_tok_s"] = round(bs / ms * 1e3, 1)
+        row[f"llama_decode_bs{bs}_ms"] = round(ms, 3)
+        del dec, mgr
+    row["llama_weight_GB"] = round(lc.weight_bytes() / 1e9, 3)
+    del model
+    torch.cuda.empty_cache()
+    return row
 
 
 def _ragged_engine_row(eng, cfg, S, prefix, kernels, width):
@@ -681,6 +700,35 @@ def fagunex_compare(args, dev):
                       "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
 
 
+def nesisun_compare(args, dev):
+    """Prefill (one prompt of --ctx tokens) and decode (bs 1 and 8 at context --ctx) of the Nesisun design through
+    InferenceEngine.run_ragged - once with dense feed-forwards of 4 x width in every layer, once with every second
+    one routed (8 experts + 1 pass-through of which 2 are used, 4 x width active) - beside the Llama-shaped runners
+    at equal width, depth and feed-forward parameters (gate, up, down of 4 x width).  Random weights, 4 layers,
+    vocabulary 32000, 128-wide heads, one key/value head per four query heads on both sides; Nesisun attends to a
+    window of 1024 and 64 kept first positions, the Llama-shaped model to everything."""
+    import micro_vllm_amd  # noqa: F401
+    from micro_vllm_amd.core.engine import InferenceEngine
+    from micro_vllm_amd.models import nesisun
+
+    S, layers, rows = args.ctx, 4, []
+    for width in [int(w) for w in args.nesisun_widths.split(",")]:
+        row = {"width": width, "layers": layers, "ctx": S}
+        for name, every in (("nesisun_dense", 0), ("nesisun_routed", 2)):
+            cfg = nesisun.bench_config(width, layers, moe_every=every)
+            eng = InferenceEngine(model=nesisun.build_random_model(cfg, seed=1), max_batch_size=8, max_prefill_tokens=S,
+                                  n_blocks=9 * (S // 64 + 4), max_tokens=S + 256, state_slots=9)
+            row.update(_ragged_engine_row(eng, cfg, S, name, args.nesisun_kernels, width))
+            del eng
+            torch.cuda.empty_cache()
+        ids = torch.randint(0, 32000, (S,), generator=torch.Generator().manual_seed(0)).tolist()
+        row.update(_llama_row(dev, width, layers, S, ids, 4 * width))
+        log(f"[bench] {row}")
+        rows.append(row)
+    print(json.dumps({"metric": "Nesisun beside the Llama-shaped family: prefill and decode tokens/s at equal size",
+                      "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
+
+
 def pagazen_kernel_table(eng, ids, width):
     """Per-op time of one prefill step and one single-token step (rocprof-free: HIP events around each
     wrapper call), printed on stderr."""
@@ -691,7 +739,8 @@ def pagazen_kernel_table(eng, ids, width):
              "softplus_decay", "scan_outer", "rotary_pairs_", "gated_group_norm", "qk_unitnorm_store", "window_attn",
              "dyt_shift", "dyt_gather", "dyt_residual", "unitnorm_residual", "rmsnorm_rows", "gelu_gate_rows", "silu_mul",
              "sigmoid_gate", "linear_heads", "linear_segments", "gate_lower_bound_", "scan_gated", "latent_prep",
-             "latent_attn", "moe_route", "moe_plan", "moe_combine"]
+             "latent_attn", "moe_route", "moe_plan", "moe_combine", "embed_pair", "add_rmsnorm", "rmsnorm_gather",
+             "gated_act", "qk_rotary_store", "moe_route_scored"]
     saved = {n: getattr(ops, n) for n in names}
     saved_call = ops.AnyLinear.__call__
 
@@ -823,6 +872,9 @@ def main():
     if args.fagunex:
         assert world == 1, "--fagunex runs on one GPU"
         return fagunex_compare(args, dev)
+    if args.nesisun:
+        assert world == 1, "--nesisun runs on one GPU"
+        return nesisun_compare(args, dev)
     peers = world > 1                 # ranks to synchronise with
     if args.as_rank_of:
         assert world == 1, "--as-rank-of runs one process"

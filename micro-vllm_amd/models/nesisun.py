@@ -174,7 +174,7 @@ def build_random_model(cfg: NesisunConfig, seed: int = 0) -> NesisunModel:
 def bench_config(width: int, n_layers: int, vocab: int = 32000, ff_mult: int = 4, window: int = 1024,
                  keep_first: int = 64, experts: int = 8, top: int = 2, moe_every: int = 2) -> NesisunConfig:
     """A configuration with the proportions of a served model: 128-wide heads, one key/value head per four query
-    heads, every `moe_every`-th layer routed (active feed-forward width ff_mult * width), the others dense."""
+    heads, every `moe_every`-th layer routed (active feed-forward width ff_mult * width; 0: none), the others dense."""
     heads = max(1, width // 128)
     mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
              "mask": {"size": window, "keep_first": keep_first}, "rot": {"base": 10000.0, "dims": 128},
@@ -183,7 +183,7 @@ def bench_config(width: int, n_layers: int, vocab: int = 32000, ff_mult: int = 4
     moe = {"kind": "moe", "expert": {"ff": eff, "limit": 7.0},
            "router": {"experts": experts, "identity": 1, "top": top, "scale": 1.0}}
     dense = {"kind": "dense", "ff": ff_mult * width}
-    layers = [{"type": "attention", "mixer": mixer, "mlp": moe if i % moe_every == moe_every - 1 else dense}
+    layers = [{"type": "attention", "mixer": mixer, "mlp": moe if moe_every and i % moe_every == moe_every - 1 else dense}
               for i in range(n_layers)]
     return NesisunConfig(vocab_size=vocab, width=width, layers=layers, embed_scale=1.0, pair_buckets=65521,
                          pair_mul_prev=1000003, pair_mul_cur=31, eps=1e-5, name=f"nesisun-w{width}-l{n_layers}")
