@@ -561,7 +561,10 @@ int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* 
 /* out[t, h*dv ..] = softmax_j( q_t . k_j * scale - slopes[h] * (pos - j) ) v_j over pos - window < j <= pos
  * from the pages (the step's own keys must already be stored).  dv <= 256.  keep_first > 0: positions below it
  * stay visible when the window has passed them, at their true positions.  sinks (fp32 [heads] or NULL): exp(sinks[h])
- * is one more term of the softmax's denominator, unscaled, with no value.  slopes NULL: no distance penalty.  With a chunk table (chunks > 0:
+ * is one more term of the softmax's denominator, unscaled, with no value.  slopes NULL: no distance penalty.
+ * part != NULL with splits >= 1 (fp32 [tokens * heads * splits * (dv + 2)]): the tokens the tiled kernel does not take
+ * run one workgroup per (token, key/value head, up to eight of its query heads, split of the keys) - every key and value
+ * is read once for those heads - and, with splits > 1, a second launch merges the splits' pieces.  With a chunk table (chunks > 0:
  * rows of more than max_len tokens cut into runs of up to 64, as for mv_scan_chunked; row_len per row), bf16
  * and a head shape the tiled kernel is built for - (d, dv) in (32,32) (64,64) (96,96) (128,128) (128,64)
  * (64,128), 64-token pages - those rows run on the matrix cores, a workgroup per (chunk, head): q.k in bf16
@@ -571,7 +574,10 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
-                   int chunks, int max_len, int keep_first, const float* sinks, mv_stream_t stream);
+                   int chunks, int max_len, int keep_first, const float* sinks, float* part, int splits,
+                   mv_stream_t stream);
+/* How many splits of the keys mv_window_attn should be given for a step of `tokens` tokens (1: none). */
+int mv_window_attn_splits(int tokens, int heads, int kv_heads, int window, int keep_first);
 
 /* ---- further row-wise steps of fp32-stream stacks (stream_ops.hip) ---------------------------------- */
 

@@ -66,14 +66,16 @@ class RaggedRunner:
     PAGE = 64
 
     def __init__(self, model, device="cuda", dtype=torch.bfloat16, wave_tiles: bool = True,
-                 chunked_scan: bool = True, graphs: bool = True, max_graph_rows: int = 64, tiled_attn: bool = True):
+                 chunked_scan: bool = True, graphs: bool = True, max_graph_rows: int = 64, tiled_attn: bool = True,
+                 grouped_attn: bool = True):
         """`wave_tiles` / `chunked_scan` = False keep every projection on the plain any-shape kernel and
         every recurrence token by token, `tiled_attn` = False every token on the plain attention kernel (the
-        forms the faster ones are checked against).  `graphs`:
+        forms the faster ones are checked against), `grouped_attn` = False the tokens of short rows on the
+        one-workgroup-per-(token, head) attention instead of the one that shares reads among query heads.  `graphs`:
         steps in which every row brings one token (decoding) are captured once per row count into a
         hipGraph and replayed - some seventy launches become one."""
         assert dtype in (torch.bfloat16, torch.float32)
-        self.chunked_scan, self.tiled_attn = chunked_scan, tiled_attn
+        self.chunked_scan, self.tiled_attn, self.grouped_attn = chunked_scan, tiled_attn, grouped_attn
         self.use_graphs, self.max_graph_rows = graphs, max_graph_rows
         self._graphs: Dict[int, tuple] = {}
         self._arena, self._arena_off, self._measured = None, 0, 0
@@ -443,8 +445,13 @@ class RaggedRunner:
         ops.qk_rotary_store(qk, w["q_b"], w["k_b"], kc, vc, w["inv_freq"], step, H, G, d, int(m["rot"]["dims"]),
                             adjacent=True)
         cat = self._actbuf(T, H * d + ff)                          # [attention output | activations]
-        ops.window_attn(qk, kc, vc, cat[:, :H * d], step, None, H, G, d, d, float(m["scale"]), int(m["mask"]["size"]),
-                        tiled=self.tiled_attn, keep_first=int(m["mask"].get("keep_first", 0)), sinks=w["sink"])
+        window, keep = int(m["mask"]["size"]), int(m["mask"].get("keep_first", 0))
+        # tokens of short rows (decoding): the query heads of a key/value head share its reads, the keys are cut over
+        # several workgroups and the pieces meet in `part`
+        splits = ops.window_attn_splits(T, H, G, window, keep) if self.grouped_attn else 0
+        part = self._f32buf(1, T * H * splits * (d + 2)) if splits else None
+        ops.window_attn(qk, kc, vc, cat[:, :H * d], step, None, H, G, d, d, float(m["scale"]), window,
+                        tiled=self.tiled_attn, keep_first=keep, sinks=w["sink"], part=part, splits=splits)
         if dense:
             ops.gated_act(proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH)
         y1 = w["w_out"](cat, self._f32buf(T, self.width))

@@ -805,6 +805,246 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
     }
 }
 
+
+// The same attention for steps of few tokens (decoding), where one workgroup per (token, head) leaves most of the chip
+// idle and every query head of a key/value head reads the same pages again: one workgroup of four waves per (token,
+// key/value head, group of up to eight of its query heads, split of the key tiles).  A wave takes 64-key tiles - those
+// of the kept first positions, then the window's - in steps of 4 * splits; a lane scores ONE key for all heads of the
+// group from one read of it, the heads' softmax pieces go through LDS, and the weighted values are gathered with
+// 16-byte loads (dv / VEC lanes per value row, several rows per load; `vec` == 0: a lane per value column).  The
+// waves' partial softmaxes meet in LDS; with splits > 1 the workgroup leaves (max, sum, weighted values) in `part`
+// for window_attn_merge_kernel, which also adds the sink.
+constexpr int kGrpMax = 8;
+
+template <bool F32, int RT>
+__global__ __launch_bounds__(256) void window_attn_group_kernel(const float* q, int64_t ldq, const void* kc_,
+                                                                const void* vc_, void* out_, int64_t ldo, float* part,
+                                                                PagedRows pr, const float* slopes, const float* sinks,
+                                                                int H, int G, int d, int dv, float scale, int window,
+                                                                int keep_first, const int* row_len, int max_len,
+                                                                int splits, int vec) {
+    typedef typename ActS<F32>::T T_;
+    constexpr int VEC = F32 ? 4 : 8;
+    extern __shared__ float lds[];
+    const T_* kc = (const T_*)kc_;
+    const T_* vc = (const T_*)vc_;
+    const int R = H / G, ngrp = (R + kGrpMax - 1) / kGrpMax;
+    const int unit = blockIdx.x, split = blockIdx.y;
+    const int t = unit / (G * ngrp), g = (unit / ngrp) % G, grp = unit % ngrp;
+    if (max_len > 0 && row_len[pr.tok_row[t]] > max_len) return;   // the tiled kernel's rows
+    const int h0 = g * R + grp * kGrpMax;
+    const int nh = R - grp * kGrpMax < kGrpMax ? R - grp * kGrpMax : kGrpMax;   // heads of this workgroup, <= RT
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
+    float* qs = lds;                    // [RT][d]
+    float* ps = qs + RT * d;            // [4][RT][64]
+    float* red = ps + 4 * RT * 64;      // [4][RT][dv]
+    float* mm = red + 4 * RT * dv;      // [4][RT]
+    float* ll = mm + 4 * RT;            // [4][RT]
+    for (int i = tid; i < RT * d; i += 256) {
+        const int r = i / d;
+        qs[i] = r < nh ? q[(int64_t)t * ldq + (int64_t)(h0 + r) * d + (i - r * d)] : 0.f;
+    }
+    __syncthreads();
+    const int pos = pr.tok_pos[t];
+    const int* bt = pr.block_table + (int64_t)pr.tok_row[t] * pr.bt_stride;
+    const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int kept = keep_first < lo ? keep_first : lo;
+    const int nk = (kept + 63) / 64, nw = (pos - lo) / 64 + 1;
+    float m[RT], l[RT], slope[RT], acc[RT][8];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+        slope[r] = (slopes && r < nh) ? slopes[h0 + r] : 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+    }
+    const int lpr = vec ? dv / VEC : 1, rp = vec ? 64 / lpr : 1;   // lanes per value row, rows per load
+    const int sub = lane / lpr, cb = lane - sub * lpr;
+    float* pw = ps + wv * RT * 64;
+    for (int u = split * 4 + wv; u < nk + nw; u += 4 * splits) {
+        const int first = u < nk ? 64 * u : lo + 64 * (u - nk);
+        const int end = u < nk ? kept - 1 : pos;
+        const int last = first + 63 < end ? first + 63 : end;
+        const int j = first + lane;
+        const bool valid = j <= last;
+        float dot[RT];
+#pragma unroll
+        for (int r = 0; r < RT; ++r) dot[r] = 0.f;
+        if (valid) {
+            const T_* kr = kc + (((int64_t)bt[j / pr.page] * pr.page + j % pr.page) * G + g) * d;
+            if (!F32 && (d & 7) == 0) {
+                for (int c = 0; c < d; c += 8) {
+                    const uint4 kv = ld16(kr + c);
+                    const float k8[8] = {bf16_lo(kv.x), bf16_hi(kv.x), bf16_lo(kv.y), bf16_hi(kv.y),
+                                         bf16_lo(kv.z), bf16_hi(kv.z), bf16_lo(kv.w), bf16_hi(kv.w)};
+#pragma unroll
+                    for (int r = 0; r < RT; ++r) {
+                        const float4 qa = *reinterpret_cast<const float4*>(qs + r * d + c);
+                        const float4 qb = *reinterpret_cast<const float4*>(qs + r * d + c + 4);
+                        dot[r] = fmaf(qa.x, k8[0], dot[r]);
+                        dot[r] = fmaf(qa.y, k8[1], dot[r]);
+                        dot[r] = fmaf(qa.z, k8[2], dot[r]);
+                        dot[r] = fmaf(qa.w, k8[3], dot[r]);
+                        dot[r] = fmaf(qb.x, k8[4], dot[r]);
+                        dot[r] = fmaf(qb.y, k8[5], dot[r]);
+                        dot[r] = fmaf(qb.z, k8[6], dot[r]);
+                        dot[r] = fmaf(qb.w, k8[7], dot[r]);
+                    }
+                }
+            } else {
+                for (int c = 0; c < d; ++c) {
+                    const float kf = ActS<F32>::ld(kr + c);
+#pragma unroll
+                    for (int r = 0; r < RT; ++r) dot[r] = fmaf(qs[r * d + c], kf, dot[r]);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const float sc = valid ? dot[r] * scale - slope[r] * (float)(pos - j) : -INFINITY;
+            const float mn = fmaxf(m[r], wave_max(sc));        // finite: a tile holds at least one key
+            const float pj = valid ? expf(sc - mn) : 0.f;
+            const float corr = expf(m[r] - mn);                // m = -inf on the wave's first tile: exp(-inf) = 0
+            l[r] = l[r] * corr + wave_sum(pj);
+            m[r] = mn;
+            pw[r * 64 + lane] = pj;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[r][e] *= corr;
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int cnt = last - first + 1;
+        if (vec) {
+            if (sub < rp) {
+                for (int row = sub; row < cnt; row += rp) {
+                    const int jk = first + row;
+                    const T_* vr = vc + (((int64_t)bt[jk / pr.page] * pr.page + jk % pr.page) * G + g) * dv + cb * VEC;
+                    const uint4 vv = ld16(vr);
+                    float v8[8];
+                    if (F32) {
+                        v8[0] = __uint_as_float(vv.x); v8[1] = __uint_as_float(vv.y);
+                        v8[2] = __uint_as_float(vv.z); v8[3] = __uint_as_float(vv.w);
+                        v8[4] = v8[5] = v8[6] = v8[7] = 0.f;
+                    } else {
+                        v8[0] = bf16_lo(vv.x); v8[1] = bf16_hi(vv.x); v8[2] = bf16_lo(vv.y); v8[3] = bf16_hi(vv.y);
+                        v8[4] = bf16_lo(vv.z); v8[5] = bf16_hi(vv.z); v8[6] = bf16_lo(vv.w); v8[7] = bf16_hi(vv.w);
+                    }
+#pragma unroll
+                    for (int r = 0; r < RT; ++r) {
+                        const float w = pw[r * 64 + row];
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[r][e] = fmaf(w, v8[e], acc[r][e]);
+                    }
+                }
+            }
+        } else {
+            for (int row = 0; row < cnt; ++row) {
+                const int jk = first + row;
+                const T_* vr = vc + (((int64_t)bt[jk / pr.page] * pr.page + jk % pr.page) * G + g) * dv;
+#pragma unroll
+                for (int ci = 0; ci < kMaxVC; ++ci) {
+                    const int c = lane + ci * 64;
+                    if (c < dv) {
+                        const float x = ActS<F32>::ld(vr + c);
+#pragma unroll
+                        for (int r = 0; r < RT; ++r) acc[r][ci] = fmaf(pw[r * 64 + row], x, acc[r][ci]);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            mm[wv * RT + r] = m[r];
+            ll[wv * RT + r] = l[r];
+        }
+    }
+    float* rw = red + wv * RT * dv;
+    if (vec) {
+        // the row groups of a wave add their sums one after the other
+        for (int s2 = 0; s2 < rp; ++s2) {
+            if (sub == s2) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const int i = r * dv + cb * VEC + e;
+                        rw[i] = (s2 == 0 ? 0.f : rw[i]) + acc[r][e];
+                    }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else {
+#pragma unroll
+        for (int ci = 0; ci < kMaxVC; ++ci) {
+            const int c = lane + ci * 64;
+            if (c < dv)
+#pragma unroll
+                for (int r = 0; r < RT; ++r) rw[r * dv + c] = acc[r][ci];
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < nh * dv; i += 256) {
+        const int r = i / dv, c = i - r * dv;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, mm[w * RT + r]);
+        float L = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = mm[w * RT + r];
+            const float f = mw == -INFINITY ? 0.f : expf(mw - M);     // a wave (or a whole split) without keys
+            L = fmaf(ll[w * RT + r], f, L);
+            o = fmaf(red[(w * RT + r) * dv + c], f, o);
+        }
+        const int h = h0 + r;
+        if (splits == 1) {
+            if (sinks) {
+                const float sk = sinks[h], mf = fmaxf(M, sk), f = expf(M - mf);
+                L = L * f + expf(sk - mf);
+                o *= f;
+            }
+            ActS<F32>::st((T_*)out_ + (int64_t)t * ldo + (int64_t)h * dv + c, o / L);
+        } else {
+            float* dst = part + (((int64_t)t * H + h) * splits + split) * (dv + 2);
+            if (c == 0) {
+                dst[0] = M;
+                dst[1] = L;
+            }
+            dst[2 + c] = o;
+        }
+    }
+}
+
+// one wave per (token, head): the splits' pieces and the sink become the output row
+template <bool F32>
+__global__ __launch_bounds__(64) void window_attn_merge_kernel(const float* part, void* out_, int64_t ldo,
+                                                               const int* tok_row, const float* sinks, int H, int dv,
+                                                               int splits, const int* row_len, int max_len) {
+    typedef typename ActS<F32>::T T_;
+    const int t = blockIdx.x / H, h = blockIdx.x % H, lane = threadIdx.x;
+    if (max_len > 0 && row_len[tok_row[t]] > max_len) return;
+    const float* src = part + (int64_t)blockIdx.x * splits * (dv + 2);
+    float M = sinks ? sinks[h] : -INFINITY;
+    for (int s2 = 0; s2 < splits; ++s2) M = fmaxf(M, src[(int64_t)s2 * (dv + 2)]);
+    float L = sinks ? expf(sinks[h] - M) : 0.f;
+    for (int s2 = 0; s2 < splits; ++s2) {
+        const float ms = src[(int64_t)s2 * (dv + 2)];
+        if (ms != -INFINITY) L = fmaf(src[(int64_t)s2 * (dv + 2) + 1], expf(ms - M), L);
+    }
+    for (int c = lane; c < dv; c += 64) {
+        float o = 0.f;
+        for (int s2 = 0; s2 < splits; ++s2) {
+            const float ms = src[(int64_t)s2 * (dv + 2)];
+            if (ms != -INFINITY) o = fmaf(src[(int64_t)s2 * (dv + 2) + 2 + c], expf(ms - M), o);
+        }
+        ActS<F32>::st((T_*)out_ + (int64_t)t * ldo + (int64_t)h * dv + c, o / L);
+    }
+}
+
 // The same attention for a prompt's portion, bf16 keys and values: one workgroup per (64 consecutive tokens
 // of a row, head).  Key tiles are pages (64 tokens) staged once in LDS for all 64 queries; q.k on
 // v_mfma_f32_16x16x32_bf16 (q rounded to bf16 as the keys are), scores, distance penalty, mask and softmax
@@ -1207,11 +1447,25 @@ int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* 
     return check_launch();
 }
 
+int mv_window_attn_splits(int tokens, int heads, int kv_heads, int window, int keep_first) {
+    using namespace mv;
+    if (tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || window <= 0 || keep_first < 0) return 1;
+    const int R = heads / kv_heads, ngrp = (R + kGrpMax - 1) / kGrpMax;
+    const int64_t units = (int64_t)tokens * kv_heads * ngrp;
+    const int64_t tiles = ((int64_t)window + keep_first) / 64 + 2;      // at most this many 64-key tiles a token
+    int64_t want = (2 * (int64_t)num_cus() + units - 1) / units;         // about two workgroups a compute unit
+    const int64_t most = (tiles + 3) / 4;                                // a wave should find a tile of its own
+    if (want > most) want = most;
+    if (want > 64) want = 64;
+    return want < 1 ? 1 : (int)want;
+}
+
 int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
-                   int chunks, int max_len, int keep_first, const float* sinks, mv_stream_t stream) {
+                   int chunks, int max_len, int keep_first, const float* sinks, float* part, int splits,
+                   mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || window <= 0 ||
         heads % kv_heads || keep_first < 0)
@@ -1242,6 +1496,35 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
         else if (d == 64 && dv == 128) { MV_WA_TILE(2, 8); }
         else if (d == 32 && dv == 32) { MV_WA_TILE(1, 2); }
 #undef MV_WA_TILE
+    }
+    // with a place for the splits' pieces: the kernel that shares every key among the query heads of its key/value
+    // head and cuts the keys over several workgroups
+    if (part && splits >= 1) {
+        const int R = heads / kv_heads, ngrp = (R + kGrpMax - 1) / kGrpMax, top = R < kGrpMax ? R : kGrpMax;
+        const int rt = top <= 1 ? 1 : top <= 2 ? 2 : top <= 4 ? 4 : 8;
+        const int vecw = f32 ? 4 : 8;
+        const int vec = dv % vecw == 0 && dv / vecw <= 64 && aligned16(v_cache);
+        const size_t glds = ((size_t)rt * d + 4 * rt * 64 + 4 * (size_t)rt * dv + 8 * rt) * sizeof(float);
+        if (glds <= 64 * 1024 && d % 4 == 0 && ldq % 4 == 0 && aligned16(q) && (f32 || d % 8 != 0 || aligned16(k_cache))) {
+            const dim3 gg((unsigned)(tokens * kv_heads * ngrp), splits);
+#define MV_WA_GROUP(F32_, RT_)                                                                                         \
+    hipLaunchKernelGGL((window_attn_group_kernel<F32_, RT_>), gg, dim3(256), glds, s, q, ldq, k_cache, v_cache, out, ldo, \
+                       part, pr, slopes, sinks, heads, kv_heads, d, dv, scale, window, keep_first, row_len, skip_len,   \
+                       splits, vec)
+            if (f32) {
+                if (rt == 1) MV_WA_GROUP(true, 1); else if (rt == 2) MV_WA_GROUP(true, 2);
+                else if (rt == 4) MV_WA_GROUP(true, 4); else MV_WA_GROUP(true, 8);
+            } else {
+                if (rt == 1) MV_WA_GROUP(false, 1); else if (rt == 2) MV_WA_GROUP(false, 2);
+                else if (rt == 4) MV_WA_GROUP(false, 4); else MV_WA_GROUP(false, 8);
+            }
+#undef MV_WA_GROUP
+            if (splits > 1) {
+                if (f32) hipLaunchKernelGGL(window_attn_merge_kernel<true>, grid, dim3(64), 0, s, part, out, ldo, tok_row, sinks, heads, dv, splits, row_len, skip_len);
+                else hipLaunchKernelGGL(window_attn_merge_kernel<false>, grid, dim3(64), 0, s, part, out, ldo, tok_row, sinks, heads, dv, splits, row_len, skip_len);
+            }
+            return check_launch();
+        }
     }
     // few (token, head) pairs and a window of many tiles: sixteen waves share it
     const bool wide = units <= 2 * num_cus() && window > 256;

@@ -243,10 +243,14 @@ def qk_rotary_store(qk, q_bias, k_bias, k_cache, v_cache, inv_freq, step, heads:
 
 
 def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: int, d: int, dv: int,
-                scale: float, window: int, tiled: bool = True, keep_first: int = 0, sinks=None):
+                scale: float, window: int, tiled: bool = True, keep_first: int = 0, sinks=None, part=None, splits: int = 0):
     """`tiled`: rows of more than SCAN_SEQ_MAX tokens go to the matrix-core kernel where it applies (bf16,
     the head shapes it is built for); False keeps every token on the plain kernel.  `keep_first`: positions below it
-    stay visible behind the window; `sinks` [heads]: exp(sink) joins each head's denominator."""
+    stay visible behind the window; `sinks` [heads]: exp(sink) joins each head's denominator.  `part` (fp32, at least
+    tokens * heads * splits * (dv + 2) values, `splits` from window_attn_splits): the tokens the matrix-core kernel
+    does not take run the kernel that reads every key once for all query heads of its key/value head and cuts the keys
+    into `splits` pieces."""
+    assert part is None or (splits >= 1 and part.is_contiguous() and part.numel() >= q.shape[0] * heads * splits * (dv + 2))
     assert sinks is None or (sinks.numel() == heads and sinks.is_contiguous())
     tokens = q.shape[0]
     assert q.shape[1] >= heads * d and out.shape == (tokens, heads * dv) and out.dtype == k_cache.dtype
@@ -261,7 +265,12 @@ def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: in
         int(window), _is_f32(k_cache), step.row_len.data_ptr(),
         step.ch_start.data_ptr() if step.n_chunks else None, step.ch_len.data_ptr() if step.n_chunks else None,
         step.n_chunks if tiled else 0, SCAN_SEQ_MAX, int(keep_first), None if sinks is None else _f32(sinks).data_ptr(),
-        nv.stream_ptr()))
+        None if part is None else _f32(part).data_ptr(), int(splits) if part is not None else 0, nv.stream_ptr()))
+
+
+def window_attn_splits(tokens: int, heads: int, kv_heads: int, window: int, keep_first: int = 0) -> int:
+    """Pieces to cut a token's keys into so that a step of few tokens still fills the chip (1: no cut)."""
+    return int(nv.lib().mv_window_attn_splits(int(tokens), heads, kv_heads, int(window), int(keep_first)))
 
 
 # ---------------------------------------------------------------------------------------------------------

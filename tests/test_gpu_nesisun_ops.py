@@ -149,8 +149,10 @@ def attn_reference(qk, qb, kb, H, G, d, rot, base, scale, window, keep, sink):
                               window, keep, s)
 
 
-def attn_run(ops, cache, sid, lo, hi, qk, qb, kb, H, G, d, rot, base, scale, window, keep, sink, dt, tiled=True):
-    """Tokens lo .. hi of sequence `sid` through bias / rotation / store and the attention kernel."""
+def attn_run(ops, cache, sid, lo, hi, qk, qb, kb, H, G, d, rot, base, scale, window, keep, sink, dt, tiled=True, splits=0):
+    """Tokens lo .. hi of sequence `sid` through bias / rotation / store and the attention kernel.  `splits` > 0: the
+    tokens of short rows take the kernel that shares reads among the query heads of a key/value head, the keys cut
+    into that many pieces (more pieces than there are tiles leave some of them empty)."""
     T = hi - lo
     st = step_of(cache, [(sid, [0] * T)])
     inv = (base ** (-2.0 * torch.arange(max(rot // 2, 1), dtype=torch.float64) / max(rot, 1))).to(DEV)
@@ -160,8 +162,9 @@ def attn_run(ops, cache, sid, lo, hi, qk, qb, kb, H, G, d, rot, base, scale, win
     kc, vc = cache.k_caches[0], cache.v_caches[0]
     ops.qk_rotary_store(x, qb.to(DEV), kb.to(DEV), kc, vc, inv, st, H, G, d, rot)
     out = torch.empty(T, H * d + 8, dtype=dt, device=DEV)[:, :H * d]
+    part = torch.full((T * H * splits * (d + 2),), float("nan"), device=DEV) if splits else None
     ops.window_attn(x, kc, vc, out, st, None, H, G, d, d, scale, window, tiled=tiled, keep_first=keep,
-                    sinks=None if sink is None else sink.to(DEV))
+                    sinks=None if sink is None else sink.to(DEV), part=part, splits=splits)
     return out.float().cpu().double().view(T, H, d)
 
 
@@ -209,6 +212,24 @@ def test_attention_whole_portions_and_decoding(ops, f32, H, G, d, rot, window, k
     assert at == T and (got - want).abs().max().item() < tol
     if f32:
         assert (got - whole).abs().max().item() < 1e-5
+    cache.free("p")
+    # the same portions with the short rows on the kernel that shares reads among query heads: uncut, cut in three,
+    # and cut as the library would choose for a step of that many tokens
+    for splits in (1, 3, None):
+        parts, at = [], 0
+        for n in [61, 2, 3, 40, 2, 17, 50] + [1] * 25:
+            sp = splits or ops.window_attn_splits(n, H, G, window, keep)
+            parts.append(attn_run(ops, cache, "g", at, at + n, *args, splits=sp))
+            at += n
+        got = torch.cat(parts)
+        assert (got - want).abs().max().item() < tol, splits
+        cache.free("g")
+    # every row short (also the first portions), so that all of it runs there; and the whole prompt at once (fp32, or
+    # with the matrix-core kernel switched off)
+    parts = [attn_run(ops, cache, "s", at, min(at + 16, T), *args, splits=2) for at in range(0, T, 16)]
+    assert (torch.cat(parts) - want).abs().max().item() < tol
+    cache.free("s")
+    assert (attn_run(ops, cache, "a", 0, T, *args, tiled=False, splits=1) - want).abs().max().item() < tol
 
 
 def dominant_case(g, T, H, G, d, rot, key, query, amp=40.0):
@@ -251,6 +272,10 @@ def test_window_edge_with_a_dominant_key(ops, query, window, keep, f32):
         first = attn_run(ops, cache, "p", 0, query, *args)
         last = attn_run(ops, cache, "p", query, T, *args)
         assert (torch.cat([first, last]) - want).abs().max().item() < tol
+        cache.free("p")
+        first = attn_run(ops, cache, "g", 0, query, *args, splits=1)
+        last = attn_run(ops, cache, "g", query, T, *args, splits=2)
+        assert (torch.cat([first, last]) - want).abs().max().item() < tol
 
 
 @pytest.mark.parametrize("f32", [True, False])
@@ -282,6 +307,12 @@ def test_kept_first_positions_with_a_dominant_key(ops, keep, window, f32):
             parts.append(attn_run(ops, cache, "p", at, at + n, *args))
             at += n
         assert at == T and (torch.cat(parts) - want).abs().max().item() < tol
+        cache.free("p")
+        parts, at = [], 0
+        for n in cuts + [T - 1 - sum(cuts)] + [1]:
+            parts.append(attn_run(ops, cache, "g", at, at + n, *args, splits=1 + at % 3))
+            at += n
+        assert (torch.cat(parts) - want).abs().max().item() < tol
 
 
 def test_far_kept_key_among_hundreds_and_heavy_sink(ops):
@@ -297,7 +328,7 @@ def test_far_kept_key_among_hundreds_and_heavy_sink(ops):
     want = attn_reference(*args[:-1])
     cache = make_cache(kv={0: (G, d, d)})
     first = attn_run(ops, cache, "p", 0, 441, *args)
-    rest = [attn_run(ops, cache, "p", t, t + 1, *args) for t in range(441, T)]
+    rest = [attn_run(ops, cache, "p", t, t + 1, *args, splits=t % 4) for t in range(441, T)]
     got = torch.cat([first] + rest)
     assert (got - want).abs().max().item() < 3e-5
     k1 = (qk[1, H * d:].double() + kb.double()).view(G, d)
@@ -308,6 +339,9 @@ def test_far_kept_key_among_hundreds_and_heavy_sink(ops):
     got = attn_run(ops, cache, "s", 0, 200, *args)
     assert (got - want[:200]).abs().max().item() < 3e-5
     assert got[150, 0].abs().max().item() < 1e-2 * got[150, 1].abs().max().item()
+    for at, splits in ((200, 1), (210, 2)):      # the sink where the waves' and the splits' pieces meet
+        late = attn_run(ops, cache, "s", at, at + 10, *args, splits=splits)
+        assert (late - want[at:at + 10]).abs().max().item() < 3e-5
     # the same through the matrix-core kernel (bf16, a shape it takes)
     H, G, d, rot = 2, 2, 64, 64
     qk, qb, kb = attn_case(g, 200, H, G, d)
