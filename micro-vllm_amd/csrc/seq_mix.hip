@@ -874,22 +874,31 @@ __global__ __launch_bounds__(256) void window_attn_group_kernel(const float* q, 
         if (valid) {
             const T_* kr = kc + (((int64_t)bt[j / pr.page] * pr.page + j % pr.page) * G + g) * d;
             if (!F32 && (d & 7) == 0) {
-                for (int c = 0; c < d; c += 8) {
-                    const uint4 kv = ld16(kr + c);
-                    const float k8[8] = {bf16_lo(kv.x), bf16_hi(kv.x), bf16_lo(kv.y), bf16_hi(kv.y),
-                                         bf16_lo(kv.z), bf16_hi(kv.z), bf16_lo(kv.w), bf16_hi(kv.w)};
+                // four 16-byte pieces of the key row in flight at a time
+                for (int c0 = 0; c0 < d; c0 += 32) {
+                    uint4 kq[4];
 #pragma unroll
-                    for (int r = 0; r < RT; ++r) {
-                        const float4 qa = *reinterpret_cast<const float4*>(qs + r * d + c);
-                        const float4 qb = *reinterpret_cast<const float4*>(qs + r * d + c + 4);
-                        dot[r] = fmaf(qa.x, k8[0], dot[r]);
-                        dot[r] = fmaf(qa.y, k8[1], dot[r]);
-                        dot[r] = fmaf(qa.z, k8[2], dot[r]);
-                        dot[r] = fmaf(qa.w, k8[3], dot[r]);
-                        dot[r] = fmaf(qb.x, k8[4], dot[r]);
-                        dot[r] = fmaf(qb.y, k8[5], dot[r]);
-                        dot[r] = fmaf(qb.z, k8[6], dot[r]);
-                        dot[r] = fmaf(qb.w, k8[7], dot[r]);
+                    for (int u = 0; u < 4; ++u) kq[u] = c0 + 8 * u < d ? ld16(kr + c0 + 8 * u) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int c = c0 + 8 * u;
+                        if (c >= d) break;
+                        const uint4 kv = kq[u];
+                        const float k8[8] = {bf16_lo(kv.x), bf16_hi(kv.x), bf16_lo(kv.y), bf16_hi(kv.y),
+                                             bf16_lo(kv.z), bf16_hi(kv.z), bf16_lo(kv.w), bf16_hi(kv.w)};
+#pragma unroll
+                        for (int r = 0; r < RT; ++r) {
+                            const float4 qa = *reinterpret_cast<const float4*>(qs + r * d + c);
+                            const float4 qb = *reinterpret_cast<const float4*>(qs + r * d + c + 4);
+                            dot[r] = fmaf(qa.x, k8[0], dot[r]);
+                            dot[r] = fmaf(qa.y, k8[1], dot[r]);
+                            dot[r] = fmaf(qa.z, k8[2], dot[r]);
+                            dot[r] = fmaf(qa.w, k8[3], dot[r]);
+                            dot[r] = fmaf(qb.x, k8[4], dot[r]);
+                            dot[r] = fmaf(qb.y, k8[5], dot[r]);
+                            dot[r] = fmaf(qb.z, k8[6], dot[r]);
+                            dot[r] = fmaf(qb.w, k8[7], dot[r]);
+                        }
                     }
                 }
             } else {
@@ -917,24 +926,40 @@ __global__ __launch_bounds__(256) void window_attn_group_kernel(const float* q, 
         const int cnt = last - first + 1;
         if (vec) {
             if (sub < rp) {
-                for (int row = sub; row < cnt; row += rp) {
-                    const int jk = first + row;
-                    const T_* vr = vc + (((int64_t)bt[jk / pr.page] * pr.page + jk % pr.page) * G + g) * dv + cb * VEC;
-                    const uint4 vv = ld16(vr);
-                    float v8[8];
-                    if (F32) {
-                        v8[0] = __uint_as_float(vv.x); v8[1] = __uint_as_float(vv.y);
-                        v8[2] = __uint_as_float(vv.z); v8[3] = __uint_as_float(vv.w);
-                        v8[4] = v8[5] = v8[6] = v8[7] = 0.f;
-                    } else {
-                        v8[0] = bf16_lo(vv.x); v8[1] = bf16_hi(vv.x); v8[2] = bf16_lo(vv.y); v8[3] = bf16_hi(vv.y);
-                        v8[4] = bf16_lo(vv.z); v8[5] = bf16_hi(vv.z); v8[6] = bf16_lo(vv.w); v8[7] = bf16_hi(vv.w);
+                // a tile of 64 keys lies in two pages at most when a page holds 64 tokens or more: their ids are looked
+                // up once; eight value rows in flight at a time
+                const int pA = first / pr.page;
+                const bool two = pr.page >= 64;
+                const int pgA = bt[pA], pgB = (two && last / pr.page != pA) ? bt[pA + 1] : pgA;
+                for (int row0 = sub; row0 < cnt; row0 += 8 * rp) {
+                    uint4 vq[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int row = row0 + u * rp;
+                        const int jk = first + (row < cnt ? row : 0);
+                        const int pg = two ? (jk / pr.page == pA ? pgA : pgB) : bt[jk / pr.page];
+                        vq[u] = ld16(vc + (((int64_t)pg * pr.page + jk % pr.page) * G + g) * dv + cb * VEC);
                     }
 #pragma unroll
-                    for (int r = 0; r < RT; ++r) {
-                        const float w = pw[r * 64 + row];
+                    for (int u = 0; u < 8; ++u) {
+                        const int row = row0 + u * rp;
+                        if (row >= cnt) break;
+                        const uint4 vv = vq[u];
+                        float v8[8];
+                        if (F32) {
+                            v8[0] = __uint_as_float(vv.x); v8[1] = __uint_as_float(vv.y);
+                            v8[2] = __uint_as_float(vv.z); v8[3] = __uint_as_float(vv.w);
+                            v8[4] = v8[5] = v8[6] = v8[7] = 0.f;
+                        } else {
+                            v8[0] = bf16_lo(vv.x); v8[1] = bf16_hi(vv.x); v8[2] = bf16_lo(vv.y); v8[3] = bf16_hi(vv.y);
+                            v8[4] = bf16_lo(vv.z); v8[5] = bf16_hi(vv.z); v8[6] = bf16_lo(vv.w); v8[7] = bf16_hi(vv.w);
+                        }
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) acc[r][e] = fmaf(w, v8[e], acc[r][e]);
+                        for (int r = 0; r < RT; ++r) {
+                            const float w = pw[r * 64 + row];
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) acc[r][e] = fmaf(w, v8[e], acc[r][e]);
+                        }
                     }
                 }
             }
@@ -1048,9 +1073,9 @@ __global__ __launch_bounds__(64) void window_attn_merge_kernel(const float* part
 // The same attention for a prompt's portion, bf16 keys and values: one workgroup per (64 consecutive tokens
 // of a row, head).  Key tiles are pages (64 tokens) staged once in LDS for all 64 queries; q.k on
 // v_mfma_f32_16x16x32_bf16 (q rounded to bf16 as the keys are), scores, distance penalty, mask and softmax
-// in fp32 per lane, and P.V on v_mfma_f32_16x16x4_f32 with P staying fp32: the score accumulators of a lane,
-// S[key 16 nt + 4 (lane / 16) + j][query lane % 16], are exactly the second operand of that instruction
-// for the four keys {16 nt + j + 4 k}, so P never leaves the registers.
+// in fp32 per lane, and P.V with every fp32 weight split exactly into three bf16 numbers, on the same bf16
+// instruction with fp32 accumulators: the score accumulators of a lane, S[key 16 nt + 4 (lane / 16) + j][query
+// lane % 16], serve as its second operand where they lie, so P never leaves the registers.
 typedef __attribute__((ext_vector_type(8))) __bf16 wa_bf16x8_t;
 
 template <int KS, int CT>
@@ -1147,15 +1172,50 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
         m = mn;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) o[ct] *= corr;
+        // P.V with P kept whole: an fp32 weight is the exact sum of three bf16 numbers (its leading 8, the next 8
+        // and the last 8 bits of the mantissa, each cut off, not rounded), the values are bf16 as cached, so three
+        // bf16 matrix instructions with fp32 accumulators form the same products as one in fp32 would - at three
+        // eighths of its cost.  The contraction index of the instruction is only a label: slot (qd, e) of both
+        // operands stands for key 32 kb + 16 (e / 4) + 4 qd + e % 4, which is where the lane's scores already lie.
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
+        for (int kb = 0; kb < 2; ++kb) {
+            uint32_t hi[4], mid[4], lo[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint16_t* vrow = &Vs[16 * nt + 4 * qd + j][r];
+            for (int e2 = 0; e2 < 4; ++e2) {       // two weights per dword
+                uint32_t h2[2], m2[2], l2[2];
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-                    o[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf16_bits_to_f32(vrow[16 * ct]), sc[nt][j], o[ct], 0, 0, 0);
+                for (int x = 0; x < 2; ++x) {
+                    const int e = 2 * e2 + x;
+                    const float pv = sc[2 * kb + e / 4][e % 4];
+                    const uint32_t hb = __float_as_uint(pv) & 0xffff0000u;
+                    const float r1 = pv - __uint_as_float(hb);
+                    const uint32_t mb = __float_as_uint(r1) & 0xffff0000u;
+                    const float r2 = r1 - __uint_as_float(mb);
+                    h2[x] = hb;
+                    m2[x] = mb;
+                    l2[x] = __float_as_uint(r2) & 0xffff0000u;
+                }
+                hi[e2] = (h2[0] >> 16) | h2[1];
+                mid[e2] = (m2[0] >> 16) | m2[1];
+                lo[e2] = (l2[0] >> 16) | l2[1];
             }
+            const wa_bf16x8_t ph = __builtin_bit_cast(wa_bf16x8_t, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+            const wa_bf16x8_t pm = __builtin_bit_cast(wa_bf16x8_t, make_uint4(mid[0], mid[1], mid[2], mid[3]));
+            const wa_bf16x8_t pl = __builtin_bit_cast(wa_bf16x8_t, make_uint4(lo[0], lo[1], lo[2], lo[3]));
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                uint32_t vw[4];
+#pragma unroll
+                for (int e2 = 0; e2 < 4; ++e2) {
+                    const int k0 = 32 * kb + 16 * (e2 / 2) + 4 * qd + 2 * (e2 % 2);
+                    vw[e2] = (uint32_t)Vs[k0][16 * ct + r] | ((uint32_t)Vs[k0 + 1][16 * ct + r] << 16);
+                }
+                const wa_bf16x8_t vf = __builtin_bit_cast(wa_bf16x8_t, make_uint4(vw[0], vw[1], vw[2], vw[3]));
+                o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, o[ct], 0, 0, 0);
+                o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pm, o[ct], 0, 0, 0);
+                o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o[ct], 0, 0, 0);
+            }
+        }
     }
     if (qok) {
         float inv = 1.0f / l;
