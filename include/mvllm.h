@@ -613,10 +613,10 @@ int mv_gated_act(const float* a, int64_t lda, void* out, int64_t ldo, int rows, 
                  float slope, int f32, mv_stream_t stream);
 /* x[r,:] = table[ids[r],:] * scale + pairs[j,:] (fp32), j = (prev[r] * mul_prev + ids[r] * mul_cur) mod buckets, or
  * j = buckets (the table's extra last row) where prev[r] < 0: the token has no predecessor.  Tables in the
- * activation type, `pairs` [buckets + 1, n]. */
+ * activation type, `pairs` [buckets + 1, n].  norm_w != NULL: h = act( x / sqrt(mean(x^2) + eps) * norm_w ) as well. */
 int mv_embed_pair(const void* table, const void* pairs, const int32_t* ids, const int32_t* prev, float* x, int64_t ldx,
-                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale, int f32,
-                  mv_stream_t stream);
+                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale,
+                  const float* norm_w, float eps, void* h, int64_t ldh, int f32, mv_stream_t stream);
 /* x += y1 (+ y2) (y1 == NULL: x as it is); w != NULL: h = act( x / sqrt(mean(x^2) + eps) * w ). */
 int mv_add_rmsnorm(const float* y1, int64_t ld1, const float* y2, int64_t ld2, float* x, int64_t ldx, const float* w,
                    float eps, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream);

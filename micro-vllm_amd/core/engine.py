@@ -203,7 +203,8 @@ class InferenceEngine:
             start += len(toks)
         want_t = torch.tensor(want, dtype=torch.int32).to(self.device, non_blocking=True) if want else \
             torch.zeros(0, dtype=torch.int32, device=self.device)
-        logits = self.runner.forward(step, self.cache_manager, want_t, residuals=residuals)
+        logits = self.runner.forward(step, self.cache_manager, want_t, residuals=residuals,
+                                     want_all=want == list(range(start)))
         self.cache_manager.advance(rows)
         return logits
 

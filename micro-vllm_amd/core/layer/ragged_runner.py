@@ -37,7 +37,8 @@ Per layer (Fagunex; norms are Dynamic Tanh, before and after each sublayer):
             x += unit-RMS * weight
 
 Per layer (Nesisun; both sublayers of a layer read ONE RMS norm and enter the stream together):
-  embedding table row * scale + row of the pair-hashed table (the token before each token comes with the step)
+  embedding table row * scale + row of the pair-hashed table (the token before each token comes with the step), and
+            the first layer's norm of it, in one launch
   attention ONE projection of h gives q | k (| gate | up of a dense feed-forward) -> biases, rotation of adjacent pairs,
             the rotated key into the key page and the key as projected into the value page (the values ARE the
             unrotated keys) -> softmax attention over the window and the kept first positions with a sink in the
@@ -313,12 +314,12 @@ class RaggedRunner:
 
     @torch.inference_mode()
     def forward(self, step: RaggedStep, cache: HybridCacheManager, want: Optional[torch.Tensor] = None,
-                residuals: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+                residuals: Optional[List[torch.Tensor]] = None, want_all: bool = False) -> torch.Tensor:
         """Run the step; returns fp32 logits [len(want), vocab] for the token indices in `want` (int32 on
-        the device; None = every token).  `residuals` receives a copy of the stream after every layer
-        run (debugging and tests)."""
+        the device; None = every token; `want_all`: the caller knows that `want` lists every token in order).
+        `residuals` receives a copy of the stream after every layer run (debugging and tests)."""
         if (self.use_graphs and residuals is None and step.tokens == step.rows <= self.max_graph_rows):
-            return self._replay(step, cache, want)
+            return self._replay(step, cache, None if want_all else want)
         return self._run(step, cache, want, residuals)
 
     # ------------------------------------------------------------------ captured decoding steps
@@ -383,8 +384,7 @@ class RaggedRunner:
         x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
         if self.parallel_prenorm:
             ops.embed_pair(self.embed, self.pair_embed, step.ids, step.tok_prev, x, cfg.embed_scale, cfg.pair_buckets,
-                           cfg.pair_mul_prev, cfg.pair_mul_cur)
-            ops.add_rmsnorm(x, w=self._w[self.runs[0][0]]["norm1"], eps=cfg.eps, h=h)
+                           cfg.pair_mul_prev, cfg.pair_mul_cur, w=self._w[self.runs[0][0]]["norm1"], eps=cfg.eps, h=h)
             for li, (wi, layer) in enumerate(self.runs):
                 y1, y2 = self._nesisun_layer(li, self._w[wi], layer, h, step, cache)
                 # both sublayers enter the stream; the next layer's norm of the new x comes out of the same launch

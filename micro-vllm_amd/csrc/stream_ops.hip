@@ -19,7 +19,8 @@
 //   silu_mul:            out = act( silu(a[:, :n]) * a[:, n:2n] )
 //   sigmoid_gate:        out = act( a * sigmoid(g) )   (g == NULL: act(a))
 //   embed_pair:          x = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets]   (a hashed
-//                        table over pairs of neighbouring tokens; row `buckets` where a token has no predecessor)
+//                        table over pairs of neighbouring tokens; row `buckets` where a token has no predecessor);
+//                        optionally h = act( x / sqrt(mean(x^2) + eps) * w ), the first layer's norm
 //   add_rmsnorm:         x += y1 (+ y2); h = act( x / sqrt(mean(x^2) + eps) * w )   (the sublayers of a parallel
 //                        layer enter the stream together and the next layer's norm comes out of the same launch)
 //   rmsnorm_gather:      out = act( x[idx] / sqrt(mean(x[idx]^2) + eps) * (offset + w) )
@@ -273,8 +274,10 @@ template <bool F32>
 __global__ __launch_bounds__(256) void embed_pair_kernel(const void* table_, const void* pairs_, const int* ids,
                                                          const int* prev, float* x, int64_t ldx, int n, int vocab,
                                                          int64_t buckets, int64_t mul_prev, int64_t mul_cur,
-                                                         float scale) {
+                                                         float scale, const float* norm_w, float eps, void* h_,
+                                                         int64_t ldh) {
     typedef typename Act<F32>::T T;
+    __shared__ float red[4];
     const T* table = (const T*)table_;
     const T* pairs = (const T*)pairs_;
     const int row = blockIdx.x;
@@ -285,8 +288,18 @@ __global__ __launch_bounds__(256) void embed_pair_kernel(const void* table_, con
     const int64_t r = pv < 0 ? buckets
                              : (((int64_t)pv % buckets) * (mul_prev % buckets) % buckets +
                                 ((int64_t)id % buckets) * (mul_cur % buckets) % buckets) % buckets;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float v = Act<F32>::ld(table + (int64_t)id * n + c) * scale + Act<F32>::ld(pairs + r * n + c);
+        x[(int64_t)row * ldx + c] = v;
+        ss += v * v;
+    }
+    if (!norm_w) return;
+    // the first layer's norm of the row out of the same launch
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
     for (int c = threadIdx.x; c < n; c += 256)
-        x[(int64_t)row * ldx + c] = Act<F32>::ld(table + (int64_t)id * n + c) * scale + Act<F32>::ld(pairs + r * n + c);
+        Act<F32>::st((T*)h_ + (int64_t)row * ldh + c, (x[(int64_t)row * ldx + c] * inv) * norm_w[c]);
 }
 
 template <bool F32>
@@ -383,16 +396,16 @@ int mv_rmsnorm_gather(const float* x, int64_t ldx, const int32_t* idx, const flo
 }
 
 int mv_embed_pair(const void* table, const void* pairs, const int32_t* ids, const int32_t* prev, float* x, int64_t ldx,
-                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale, int f32,
-                  mv_stream_t stream) {
+                  int rows, int n, int vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur, float scale,
+                  const float* norm_w, float eps, void* h, int64_t ldh, int f32, mv_stream_t stream) {
     using namespace mv;
     if (rows < 0 || n <= 0 || vocab <= 0 || buckets <= 0 || buckets > 0x7fffffff || mul_prev < 0 || mul_cur < 0)
         return MV_ERR_INVALID_ARG;
     if (rows == 0) return MV_OK;
-    if (!table || !pairs || !ids || !prev || !x || ldx < n) return MV_ERR_INVALID_ARG;
+    if (!table || !pairs || !ids || !prev || !x || ldx < n || (norm_w && (!h || ldh < n))) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(embed_pair_kernel<true>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale);
-    else hipLaunchKernelGGL(embed_pair_kernel<false>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale);
+    if (f32) hipLaunchKernelGGL(embed_pair_kernel<true>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale, norm_w, eps, h, ldh);
+    else hipLaunchKernelGGL(embed_pair_kernel<false>, dim3(rows), dim3(256), 0, s, table, pairs, ids, prev, x, ldx, n, vocab, buckets, mul_prev, mul_cur, scale, norm_w, eps, h, ldh);
     return check_launch();
 }
 

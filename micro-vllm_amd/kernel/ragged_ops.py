@@ -538,16 +538,21 @@ def gated_act(a, out, kind: int, limit: float = 0.0, slope: float = 1.0):
         _is_f32(out), nv.stream_ptr()))
 
 
-def embed_pair(table, pairs, ids, prev, x, scale: float, buckets: int, mul_prev: int, mul_cur: int):
-    """x = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets], row `buckets` where prev < 0."""
+def embed_pair(table, pairs, ids, prev, x, scale: float, buckets: int, mul_prev: int, mul_cur: int, w=None,
+               eps: float = 0.0, h=None):
+    """x = table[id] * scale + pairs[(prev * mul_prev + id * mul_cur) mod buckets], row `buckets` where prev < 0.
+    With `w`: h = act(x / sqrt(mean(x^2) + eps) * w) out of the same launch."""
     rows, n = x.shape
+    assert (w is None) == (h is None) and (w is None or (w.numel() == n and w.is_contiguous() and h.shape == (rows, n)
+                                                        and h.dtype == table.dtype))
     assert table.is_cuda and table.is_contiguous() and table.shape[1] == n and table.dtype == pairs.dtype
     assert pairs.is_cuda and pairs.is_contiguous() and pairs.shape == (buckets + 1, n)
     assert ids.numel() == rows and prev.numel() == rows
     nv.check("mv_embed_pair", nv.lib().mv_embed_pair(
         table.data_ptr(), pairs.data_ptr(), _i32(ids).data_ptr(), _i32(prev).data_ptr(), _f32(x).data_ptr(), _ld(x),
-        rows, n, table.shape[0], int(buckets), int(mul_prev), int(mul_cur), float(scale), _is_f32(table),
-        nv.stream_ptr()))
+        rows, n, table.shape[0], int(buckets), int(mul_prev), int(mul_cur), float(scale),
+        None if w is None else _f32(w).data_ptr(), float(eps), None if h is None else h.data_ptr(),
+        0 if h is None else _ld(h), _is_f32(table), nv.stream_ptr()))
 
 
 def add_rmsnorm(x, y1=None, y2=None, w=None, eps: float = 0.0, h=None):

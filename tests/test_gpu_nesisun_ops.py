@@ -62,6 +62,15 @@ def test_pair_hashed_embedding_over_steps(ops, f32, buckets, mul_prev, mul_cur):
     for k, toks in seqs.items():
         want = ref.pair_embedding(toks, embed.double(), table.double(), 2.5, buckets, mul_prev, mul_cur)
         assert (torch.cat(got[k]) - want).abs().max().item() < 1e-6, k
+    # with the first layer's norm out of the same launch
+    w = 1.0 + 0.2 * torch.randn(n, generator=g)
+    ids = torch.tensor(seqs["a"], dtype=torch.int32, device=DEV)
+    prev = torch.tensor([-1] + seqs["a"][:-1], dtype=torch.int32, device=DEV)
+    x, h = torch.empty(40, n, device=DEV), torch.empty(40, n, dtype=dt, device=DEV)
+    ops.embed_pair(embed.to(DEV), table.to(DEV), ids, prev, x, 2.5, buckets, mul_prev, mul_cur, w=w.to(DEV), eps=1e-5, h=h)
+    want = ref.pair_embedding(seqs["a"], embed.double(), table.double(), 2.5, buckets, mul_prev, mul_cur)
+    assert (x.cpu().double() - want).abs().max().item() < 1e-6
+    assert (h.float().cpu().double() - ref.rms_norm(want, w.double(), 1e-5)).abs().max().item() < (1e-5 if f32 else 3e-2)
     # a sequence that ends gives its slot to the next one, which starts without a predecessor
     cache.free("c")
     st = step_of(cache, [("d", [7, 8])])
