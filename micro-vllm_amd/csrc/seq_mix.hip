@@ -1086,7 +1086,9 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
                                                                int window, int keep_first, const float* sinks) {
     constexpr int D = KS * 32, DV = CT * 16, SK = D + 8, SV = DV + 8;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[64][SK];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[64][SV];
+    // values as pairs of neighbouring keys: dword [i][c] = V[2i][c] | V[2i+1][c] << 16, which is how the matrix
+    // instruction wants them (two contraction slots per register)
+    __shared__ __attribute__((aligned(16))) uint32_t Vp[32][SV];
     const int ch = blockIdx.x, h = blockIdx.y, g = h / (H / G);
     const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r = lane & 15, qd = lane >> 4;
     const int start = ch_start[ch], len = ch_len[ch];
@@ -1125,9 +1127,14 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
             const int rr = i / (D / 8), cc = i % (D / 8);
             st16(&Ks[rr][cc * 8], ld16(kc + ((pgrow + rr) * G + g) * D + cc * 8));
         }
-        for (int i = tid; i < 64 * (DV / 8); i += 256) {
+        for (int i = tid; i < 32 * (DV / 8); i += 256) {
             const int rr = i / (DV / 8), cc = i % (DV / 8);
-            st16(&Vs[rr][cc * 8], ld16(vc + ((pgrow + rr) * G + g) * DV + cc * 8));
+            const uint4 a = ld16(vc + ((pgrow + 2 * rr) * G + g) * DV + cc * 8);
+            const uint4 b = ld16(vc + ((pgrow + 2 * rr + 1) * G + g) * DV + cc * 8);
+            st16(&Vp[rr][cc * 8], make_uint4((a.x & 0xffffu) | (b.x << 16), (a.x >> 16) | (b.x & 0xffff0000u),
+                                             (a.y & 0xffffu) | (b.y << 16), (a.y >> 16) | (b.y & 0xffff0000u)));
+            st16(&Vp[rr][cc * 8 + 4], make_uint4((a.z & 0xffffu) | (b.z << 16), (a.z >> 16) | (b.z & 0xffff0000u),
+                                                 (a.w & 0xffffu) | (b.w << 16), (a.w >> 16) | (b.w & 0xffff0000u)));
         }
         __syncthreads();
         // nothing of this tile is visible to the wave
@@ -1156,13 +1163,14 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m, mx);
-        const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+        constexpr float kLog2e = 1.4426950408889634f;      // e^x as 2^(x log2 e) on the hardware's exp2
+        const float corr = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m - mn) * kLog2e);
         float ps = 0.f;
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float pv = sc[nt][j] == -INFINITY ? 0.f : expf(sc[nt][j] - mn);
+                const float pv = sc[nt][j] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((sc[nt][j] - mn) * kLog2e);
                 sc[nt][j] = pv;
                 ps += pv;
             }
@@ -1206,10 +1214,8 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, i
             for (int ct = 0; ct < CT; ++ct) {
                 uint32_t vw[4];
 #pragma unroll
-                for (int e2 = 0; e2 < 4; ++e2) {
-                    const int k0 = 32 * kb + 16 * (e2 / 2) + 4 * qd + 2 * (e2 % 2);
-                    vw[e2] = (uint32_t)Vs[k0][16 * ct + r] | ((uint32_t)Vs[k0 + 1][16 * ct + r] << 16);
-                }
+                for (int e2 = 0; e2 < 4; ++e2)     // keys k0, k0 + 1 with k0 = 32 kb + 16 (e2 / 2) + 4 qd + 2 (e2 % 2)
+                    vw[e2] = Vp[16 * kb + 8 * (e2 / 2) + 2 * qd + (e2 % 2)][16 * ct + r];
                 const wa_bf16x8_t vf = __builtin_bit_cast(wa_bf16x8_t, make_uint4(vw[0], vw[1], vw[2], vw[3]));
                 o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, o[ct], 0, 0, 0);
                 o[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pm, o[ct], 0, 0, 0);
