@@ -564,7 +564,9 @@ int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* 
  * is one more term of the softmax's denominator, unscaled, with no value.  slopes NULL: no distance penalty.
  * part != NULL with splits >= 1 (fp32 [tokens * heads * splits * (dv + 2)]): the tokens the tiled kernel does not take
  * run one workgroup per (token, key/value head, up to eight of its query heads, split of the keys) - every key and value
- * is read once for those heads - and, with splits > 1, a second launch merges the splits' pieces.  With a chunk table (chunks > 0:
+ * is read once for those heads - and, with splits > 1, a second launch merges the splits' pieces.
+ * short_tokens: how many of the step's tokens lie in rows of up to max_len tokens (-1: not known); 0 lets a step whose
+ * rows all went to the tiled kernel skip the launch of the per-token form.  With a chunk table (chunks > 0:
  * rows of more than max_len tokens cut into runs of up to 64, as for mv_scan_chunked; row_len per row), bf16
  * and a head shape the tiled kernel is built for - (d, dv) in (32,32) (64,64) (96,96) (128,128) (128,64)
  * (64,128), 64-token pages - those rows run on the matrix cores, a workgroup per (chunk, head): q.k in bf16
@@ -575,7 +577,7 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
                    int chunks, int max_len, int keep_first, const float* sinks, float* part, int splits,
-                   mv_stream_t stream);
+                   int short_tokens, mv_stream_t stream);
 /* How many splits of the keys mv_window_attn should be given for a step of `tokens` tokens (1: none). */
 int mv_window_attn_splits(int tokens, int heads, int kv_heads, int window, int keep_first);
 

@@ -42,6 +42,7 @@ class RaggedStep:
     row_ch0: torch.Tensor = None    # int32 [B] the row's first chunk
     row_nch: torch.Tensor = None    # int32 [B] its number of chunks (0: a short row)
     slots: tuple = ()               # host copy of row_slot
+    short_tokens: int = -1          # tokens in rows of up to SCAN_SEQ_MAX tokens (the rows outside the chunk table); -1: unknown
 
 
 from ..kernel.ragged_ops import SCAN_SEQ_MAX  # noqa: E402  rows up to this length are not cut into chunks
@@ -229,4 +230,5 @@ class HybridCacheManager:
             row_ctx=dev[o_rows + 2 * B:o_rows + 3 * B], row_slot=dev[o_rows + 3 * B:o_rows + 4 * B],
             block_table=dev[o_bt:o_bt + B * W].view(B, W), max_slot=max_slot, max_page=max_page, n_chunks=NC,
             ch_start=dev[o_cs:o_cs + NC], ch_len=dev[o_cl:o_cl + NC], row_ch0=dev[o_c0:o_c0 + B],
-            row_nch=dev[o_nch:o_nch + B], slots=tuple(self._slot[sid] for sid, _ in rows))
+            row_nch=dev[o_nch:o_nch + B], slots=tuple(self._slot[sid] for sid, _ in rows),
+            short_tokens=sum(len(t) for _, t in rows if len(t) <= SCAN_SEQ_MAX))

@@ -1531,7 +1531,7 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
                    int chunks, int max_len, int keep_first, const float* sinks, float* part, int splits,
-                   mv_stream_t stream) {
+                   int short_tokens, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || window <= 0 ||
         heads % kv_heads || keep_first < 0)
@@ -1562,6 +1562,8 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
         else if (d == 64 && dv == 128) { MV_WA_TILE(2, 8); }
         else if (d == 32 && dv == 32) { MV_WA_TILE(1, 2); }
 #undef MV_WA_TILE
+        // every row of the step was long enough for the tiles: nothing is left for the per-token forms
+        if (skip_len > 0 && short_tokens == 0) return check_launch();
     }
     // with a place for the splits' pieces: the kernel that shares every key among the query heads of its key/value
     // head and cuts the keys over several workgroups

@@ -265,7 +265,8 @@ def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: in
         int(window), _is_f32(k_cache), step.row_len.data_ptr(),
         step.ch_start.data_ptr() if step.n_chunks else None, step.ch_len.data_ptr() if step.n_chunks else None,
         step.n_chunks if tiled else 0, SCAN_SEQ_MAX, int(keep_first), None if sinks is None else _f32(sinks).data_ptr(),
-        None if part is None else _f32(part).data_ptr(), int(splits) if part is not None else 0, nv.stream_ptr()))
+        None if part is None else _f32(part).data_ptr(), int(splits) if part is not None else 0,
+        int(getattr(step, "short_tokens", -1)) if tiled else -1, nv.stream_ptr()))
 
 
 def window_attn_splits(tokens: int, heads: int, kv_heads: int, window: int, keep_first: int = 0) -> int:

@@ -97,6 +97,14 @@ def test_step_plan_carries_the_token_before_each_token(mv):
     c.reserve([("b", 1)])
     st = c.plan([("b", [78])])
     assert st.tok_prev.tolist() == [1]
+    # tokens in rows short enough to stay outside the chunk table (the attention's per-token form serves them)
+    c.free("b")
+    c.free("c")
+    c.reserve([("x", 40), ("y", 3)])
+    assert c.plan([("x", [1] * 40), ("y", [2] * 3)]).short_tokens == 3
+    c.advance([("x", 40), ("y", 3)])
+    c.reserve([("x", 20)])
+    assert c.plan([("x", [1] * 20)]).short_tokens == 0
 
 
 def test_restatement_visibility_sink_and_values():
