@@ -552,11 +552,14 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
 /* Rows of qk are [heads x d | kv_heads x d] fp32, one projection's output.  Queries: q += q_bias (NULL: none), then
  * the first `rot` dimensions of each head rotated by angle pos * inv_freq[i] (fp64 table of rot/2 entries; adjacent:
  * dimension 2i with 2i+1, else i with i + rot/2), in place.  Keys: k += k_bias; the key as it then stands goes to
- * v_cache (attention whose values are its unrotated keys), its rotated form to k_cache, both [pages, page, kv_heads, d]. */
+ * v_cache (attention whose values are its unrotated keys), its rotated form to k_cache, both [pages, page, kv_heads, d].
+ * act_in != NULL: the same launch also forms act_out[t, :act_n] = mv_gated_act of act_in[t, :2 act_n] (gate | up columns
+ * that the same projection left beside q and k: a layer whose mixer and feed-forward read one input). */
 int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* k_bias, void* k_cache, void* v_cache,
                        const double* inv_freq, const int32_t* tok_row, const int32_t* tok_pos,
                        const int32_t* block_table, int bt_stride, int page, int tokens, int heads, int kv_heads, int d,
-                       int rot, int adjacent, int f32, mv_stream_t stream);
+                       int rot, int adjacent, const float* act_in, int64_t lda, void* act_out, int64_t ldao, int act_n,
+                       int act_kind, float act_limit, float act_slope, int f32, mv_stream_t stream);
 
 /* out[t, h*dv ..] = softmax_j( q_t . k_j * scale - slopes[h] * (pos - j) ) v_j over pos - window < j <= pos
  * from the pages (the step's own keys must already be stored).  dv <= 256.  keep_first > 0: positions below it

@@ -110,7 +110,8 @@ PROTOTYPES = {
     "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                             _P, _P, _P, _I, _I, _I, _P, _P, _I, _I, _P]),
     "mv_window_attn_splits": (_I, [_I, _I, _I, _I, _I]),
-    "mv_qk_rotary_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "mv_qk_rotary_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _P, _L,
+                                _I, _I, _F, _F, _I, _P]),
     "mv_gated_act": (_I, [_P, _L, _P, _L, _I, _I, _I, _F, _F, _I, _P]),
     "mv_embed_pair": (_I, [_P, _P, _P, _P, _P, _L, _I, _I, _I, _L, _L, _L, _F, _P, _F, _P, _L, _I, _P]),
     "mv_add_rmsnorm": (_I, [_P, _L, _P, _L, _P, _L, _P, _F, _P, _L, _I, _I, _I, _P]),

@@ -41,9 +41,9 @@ Per layer (Nesisun; both sublayers of a layer read ONE RMS norm and enter the st
             the first layer's norm of it, in one launch
   attention ONE projection of h gives q | k (| gate | up of a dense feed-forward) -> biases, rotation of adjacent pairs,
             the rotated key into the key page and the key as projected into the value page (the values ARE the
-            unrotated keys) -> softmax attention over the window and the kept first positions with a sink in the
+            unrotated keys), and in the same launch the dense feed-forward's gelu_tanh(gate) * up -> softmax attention over the window and the kept first positions with a sink in the
             denominator, written beside the feed-forward's activations
-  dense     gelu_tanh(gate) * up lands next to the attention output; ONE projection over [attention | activations]
+  dense     its activations land next to the attention output; ONE projection over [attention | activations]
             with [W_o | W_down] gives mixer + feed-forward
   moe       router (fp32 softmax over all outputs, correction for the choice only, renormalised weights) -> pairs
             sorted by expert -> gate|up by segment -> clamped gate -> down by segment -> weighted sum, a choice of
@@ -442,9 +442,11 @@ class RaggedRunner:
         proj = w["w_in"](h, self._f32buf(T, w["w_in"].n))          # [q | k (| gate | up)]
         qk = proj[:, :(H + G) * d]
         kc, vc = cache.k_caches[li], cache.v_caches[li]
-        ops.qk_rotary_store(qk, w["q_b"], w["k_b"], kc, vc, w["inv_freq"], step, H, G, d, int(m["rot"]["dims"]),
-                            adjacent=True)
         cat = self._actbuf(T, H * d + ff)                          # [attention output | activations]
+        # gelu_tanh(gate) * up lands next to where the attention output will go, out of the rotation's launch
+        ops.qk_rotary_store(qk, w["q_b"], w["k_b"], kc, vc, w["inv_freq"], step, H, G, d, int(m["rot"]["dims"]),
+                            adjacent=True,
+                            act=(proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH, 0.0, 1.0) if dense else None)
         window, keep = int(m["mask"]["size"]), int(m["mask"].get("keep_first", 0))
         # tokens of short rows (decoding): the query heads of a key/value head share its reads, the keys are cut over
         # several workgroups and the pieces meet in `part`
@@ -452,8 +454,6 @@ class RaggedRunner:
         part = self._f32buf(1, T * H * splits * (d + 2)) if splits else None
         ops.window_attn(qk, kc, vc, cat[:, :H * d], step, None, H, G, d, d, float(m["scale"]), window,
                         tiled=self.tiled_attn, keep_first=keep, sinks=w["sink"], part=part, splits=splits)
-        if dense:
-            ops.gated_act(proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH)
         y1 = w["w_out"](cat, self._f32buf(T, self.width))
         if not mlp or dense:
             return y1, None

@@ -49,6 +49,20 @@ __device__ __forceinline__ float silu_mul_rounded(float gate_acc, float up_acc) 
     return (g * sig) * u;
 }
 
+// GELU in its tanh form, and the gate of a gated feed-forward: kind 0 silu(g) u, 1 gelu_tanh(g) u, 2 the clamped
+// form g' sigmoid(slope g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit)
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    const float inner = 0.7978845608028654f * fmaf(0.044715f * z * z, z, z);
+    return 0.5f * z * (1.0f + tanhf(inner));
+}
+__device__ __forceinline__ float gated_act_f(float g, float u, int kind, float limit, float slope) {
+    if (kind == 0) return (g / (1.0f + expf(-g))) * u;
+    if (kind == 1) return gelu_tanh_f(g) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return (g / (1.0f + expf(-slope * g))) * (u + 1.0f);
+}
+
 // ---- cross-lane ----------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

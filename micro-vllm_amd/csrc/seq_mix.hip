@@ -617,8 +617,21 @@ template <bool F32>
 __global__ __launch_bounds__(256) void qk_rotary_store_kernel(float* qk, int64_t ld, const float* qb, const float* kb,
                                                               void* kc_, void* vc_, const double* inv_freq,
                                                               PagedRows pr, int T, int H, int G, int d, int rot,
-                                                              int adjacent) {
+                                                              int adjacent, unsigned rot_blocks, const float* act_in,
+                                                              int64_t lda, void* act_out, int64_t ldao, int act_n,
+                                                              int act_kind, float act_limit, float act_slope) {
     typedef typename ActS<F32>::T T_;
+    if (blockIdx.x >= rot_blocks) {
+        // the workgroups behind the rotation's: the gate of a feed-forward whose gate | up columns came out of the
+        // same projection (a parallel layer), so that the step needs no launch of its own
+        const unsigned b = blockIdx.x - rot_blocks, cb = (act_n + 255) / 256;
+        const int64_t row = b / cb;
+        const int c = (b % cb) * 256 + threadIdx.x;
+        if (c < act_n)
+            ActS<F32>::st((T_*)act_out + row * ldao + c,
+                          gated_act_f(act_in[row * lda + c], act_in[row * lda + act_n + c], act_kind, act_limit, act_slope));
+        return;
+    }
     T_* kc = (T_*)kc_;
     T_* vc = (T_*)vc_;
     const int per = H + G;
@@ -1496,9 +1509,12 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
 int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* k_bias, void* k_cache, void* v_cache,
                        const double* inv_freq, const int32_t* tok_row, const int32_t* tok_pos,
                        const int32_t* block_table, int bt_stride, int page, int tokens, int heads, int kv_heads, int d,
-                       int rot, int adjacent, int f32, mv_stream_t stream) {
+                       int rot, int adjacent, const float* act_in, int64_t lda, void* act_out, int64_t ldao, int act_n,
+                       int act_kind, float act_limit, float act_slope, int f32, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || page <= 0 || rot < 0 || rot > d || rot % 2)
+        return MV_ERR_INVALID_ARG;
+    if (act_in && (!act_out || act_n <= 0 || lda < 2 * (int64_t)act_n || ldao < act_n || act_kind < 0 || act_kind > 2))
         return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
     if (!qk || !k_cache || !v_cache || (rot > 0 && !inv_freq) || !tok_row || !tok_pos || !block_table ||
@@ -1506,10 +1522,12 @@ int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* 
         return MV_ERR_INVALID_ARG;
     PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
     const int64_t units = (int64_t)tokens * (heads + kv_heads);
-    const dim3 grid((unsigned)((units + 3) / 4));
+    const int64_t rot_blocks = (units + 3) / 4, act_blocks = act_in ? (int64_t)tokens * ((act_n + 255) / 256) : 0;
+    if (rot_blocks + act_blocks > 0x7fffffff) return MV_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)(rot_blocks + act_blocks));
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(qk_rotary_store_kernel<true>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent);
-    else hipLaunchKernelGGL(qk_rotary_store_kernel<false>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent);
+    if (f32) hipLaunchKernelGGL(qk_rotary_store_kernel<true>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
+    else hipLaunchKernelGGL(qk_rotary_store_kernel<false>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
     return check_launch();
 }
 

@@ -223,11 +223,6 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* v, int64
     for (int c = lane; c < n; c += 64) Act<F32>::st(o + c, (a[c] * inv) * w[c]);
 }
 
-__device__ __forceinline__ float gelu_tanh_f(float z) {
-    const float inner = 0.7978845608028654f * fmaf(0.044715f * z * z, z, z);
-    return 0.5f * z * (1.0f + tanhf(inner));
-}
-
 template <bool F32>
 __global__ __launch_bounds__(256) void gelu_gate_rows_kernel(const float* a, int64_t lda, const void* table_,
                                                              int64_t ldt, int off, const int* ids, int vocab,
@@ -336,17 +331,7 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const float* a, int64_t 
     const int64_t row = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= n) return;
-    float g = a[row * lda + c], u = a[row * lda + n + c], v;
-    if (kind == 0) {
-        v = (g / (1.0f + expf(-g))) * u;
-    } else if (kind == 1) {
-        v = gelu_tanh_f(g) * u;
-    } else {
-        g = fminf(g, limit);
-        u = fminf(fmaxf(u, -limit), limit);
-        v = (g / (1.0f + expf(-slope * g))) * (u + 1.0f);
-    }
-    Act<F32>::st(out + row * ldo + c, v);
+    Act<F32>::st(out + row * ldo + c, gated_act_f(a[row * lda + c], a[row * lda + n + c], kind, limit, slope));
 }
 
 }  // namespace mv

@@ -221,11 +221,19 @@ def qk_unitnorm_store(qkv, k_cache, v_cache, step, heads: int, kv_heads: int, d:
 
 
 def qk_rotary_store(qk, q_bias, k_bias, k_cache, v_cache, inv_freq, step, heads: int, kv_heads: int, d: int, rot: int,
-                    adjacent: bool = True):
+                    adjacent: bool = True, act=None):
     """qk [T, (heads + kv_heads) * d] fp32 = queries then keys of one projection.  Biases are added, queries rotated
     in place; a key goes rotated into k_cache and as projected (with its bias) into v_cache: the values of this
-    attention are its unrotated keys."""
+    attention are its unrotated keys.  `act` = (a [T, 2n] fp32, out [T, n], kind, limit, slope): the gated activation
+    of gated_act in the same launch (a feed-forward whose gate | up columns the same projection produced)."""
     tokens = qk.shape[0]
+    a_in = a_out = None
+    n_act = kind = 0
+    limit = slope = 0.0
+    if act is not None:
+        a_in, a_out, kind, limit, slope = act
+        n_act = a_out.shape[1]
+        assert a_in.shape == (tokens, 2 * n_act) and a_out.shape[0] == tokens and a_out.dtype == k_cache.dtype
     assert qk.shape[1] == (heads + kv_heads) * d and step.tokens == tokens
     page = k_cache.shape[1]
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype
@@ -239,7 +247,9 @@ def qk_rotary_store(qk, q_bias, k_bias, k_cache, v_cache, inv_freq, step, heads:
         None if k_bias is None else _f32(k_bias).data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
         None if rot == 0 else inv_freq.data_ptr(), step.tok_row.data_ptr(), step.tok_pos.data_ptr(),
         step.block_table.data_ptr(), step.block_table.stride(0), page, tokens, heads, kv_heads, d, rot, int(adjacent),
-        _is_f32(k_cache), nv.stream_ptr()))
+        None if a_in is None else _f32(a_in).data_ptr(), 0 if a_in is None else _ld(a_in),
+        None if a_in is None else a_out.data_ptr(), 0 if a_in is None else _ld(a_out), int(n_act), int(kind), float(limit),
+        float(slope), _is_f32(k_cache), nv.stream_ptr()))
 
 
 def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: int, d: int, dv: int,

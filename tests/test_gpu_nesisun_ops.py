@@ -377,6 +377,25 @@ def test_values_are_the_keys_before_rotation(ops):
     assert (vals - k).abs().max().item() < 1e-6
     assert (keys - ref.rotate_adjacent(k, torch.arange(T), rot, base)).abs().max().item() < 1e-5
     assert (keys[5] - vals[5]).abs().max().item() > 0.1 and torch.equal(keys[:, :, rot:], vals[:, :, rot:])
+    # the same launch with a feed-forward's gate | up columns behind q and k: both results as from separate launches
+    ff = 150
+    for dt in (torch.float32, torch.bfloat16):
+        c2 = make_cache(kv={0: (G, d, d)}, dtype=dt)
+        st = step_of(c2, [("x", [0] * T)])
+        inv = (base ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / rot)).to(DEV)
+        proj = torch.cat([qk, torch.randn(T, 2 * ff, generator=g) * 3], dim=1).to(DEV)
+        both, alone = torch.empty(T, 8 + ff, dtype=dt, device=DEV)[:, 8:], torch.empty(T, ff, dtype=dt, device=DEV)
+        ops.gated_act(proj[:, (H + G) * d:], alone, ops.GATE_GELU_TANH)
+        x = proj.clone()
+        ops.qk_rotary_store(x[:, :(H + G) * d], qb.to(DEV), kb.to(DEV), c2.k_caches[0], c2.v_caches[0], inv, st, H, G, d, rot,
+                            act=(x[:, (H + G) * d:], both, ops.GATE_GELU_TANH, 0.0, 1.0))
+        assert torch.equal(both, alone)
+        pg = c2.get_blocks("x")
+        k2 = torch.cat([c2.k_caches[0][p] for p in pg])[:T].float().cpu().double()
+        assert (k2 - ref.rotate_adjacent(k, torch.arange(T), rot, base)).abs().max().item() < (1e-5 if dt == torch.float32 else 3e-2)
+        q2 = x[:, :H * d].cpu().double().view(T, H, d)
+        qw = ref.rotate_adjacent((qk[:, :H * d].double() + qb.double()).view(T, H, d), torch.arange(T), rot, base)
+        assert (q2 - qw).abs().max().item() < 1e-5
 
 
 # ---------------------------------------------------------------------------------------------------- experts
