@@ -610,14 +610,14 @@ __global__ __launch_bounds__(256) void qk_unitnorm_store_kernel(float* qkv, int6
     }
 }
 
-// One wave per (token, query or key head).  q [T, ld]: heads * d query values then kv_heads * d key values, as
-// one projection leaves them.  The query gets its bias and rotation in place; the key goes, with its bias, unrotated
+// One wave per (token, `hpw` consecutive query or key heads: the sines and cosines of a position are formed once for
+// them).  q [T, ld]: heads * d query values then kv_heads * d key values, as one projection leaves them.  The query gets its bias and rotation in place; the key goes, with its bias, unrotated
 // into the value page and rotated into the key page.  angle = position * inv_freq[i], formed in fp64.
 template <bool F32>
 __global__ __launch_bounds__(256) void qk_rotary_store_kernel(float* qk, int64_t ld, const float* qb, const float* kb,
                                                               void* kc_, void* vc_, const double* inv_freq,
                                                               PagedRows pr, int T, int H, int G, int d, int rot,
-                                                              int adjacent, unsigned rot_blocks, const float* act_in,
+                                                              int adjacent, int hpw, unsigned rot_blocks, const float* act_in,
                                                               int64_t lda, void* act_out, int64_t ldao, int act_n,
                                                               int act_kind, float act_limit, float act_slope) {
     typedef typename ActS<F32>::T T_;
@@ -634,47 +634,52 @@ __global__ __launch_bounds__(256) void qk_rotary_store_kernel(float* qk, int64_t
     }
     T_* kc = (T_*)kc_;
     T_* vc = (T_*)vc_;
-    const int per = H + G;
+    const int per = H + G, groups = (per + hpw - 1) / hpw;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    if (unit >= (int64_t)T * per) return;
-    const int t = (int)(unit / per), u = (int)(unit % per);
+    if (unit >= (int64_t)T * groups) return;
+    const int t = (int)(unit / groups), u0 = (int)(unit % groups) * hpw, u1 = u0 + hpw < per ? u0 + hpw : per;
     const int pos = pr.tok_pos[t];
-    float* p = qk + (int64_t)t * ld + (int64_t)u * d;
-    const float* bias = u < H ? (qb ? qb + (int64_t)u * d : nullptr) : (kb ? kb + (int64_t)(u - H) * d : nullptr);
-    T_* kdst = nullptr;
-    T_* vdst = nullptr;
-    if (u >= H) {
+    float* row = qk + (int64_t)t * ld;
+    int64_t slot = -1;            // the token's place in the pages (needed where the wave holds a key head)
+    if (u1 > H) {
         const int pg = pr.block_table[(int64_t)pr.tok_row[t] * pr.bt_stride + pos / pr.page];
-        if (pg < 0) return;
-        const int64_t slot = ((int64_t)pg * pr.page + pos % pr.page) * G + (u - H);
-        kdst = kc + slot * d;
-        vdst = vc + slot * d;
+        if (pg >= 0) slot = ((int64_t)pg * pr.page + pos % pr.page) * G;
     }
     const int half = rot / 2;
     for (int i = lane; i < half; i += 64) {
         const int a = adjacent ? 2 * i : i, b = adjacent ? 2 * i + 1 : i + half;
         const double ang = (double)pos * inv_freq[i];
-        const float cs = (float)cos(ang), sn = (float)sin(ang);
-        const float x0 = bias ? p[a] + bias[a] : p[a], x1 = bias ? p[b] + bias[b] : p[b];
-        const float r0 = x0 * cs - x1 * sn, r1 = x1 * cs + x0 * sn;
-        if (u < H) {
-            p[a] = r0;
-            p[b] = r1;
-        } else {
-            ActS<F32>::st(kdst + a, r0);
-            ActS<F32>::st(kdst + b, r1);
-            ActS<F32>::st(vdst + a, x0);
-            ActS<F32>::st(vdst + b, x1);
+        const float cs = (float)cos(ang), sn = (float)sin(ang);     // once for all heads of the wave
+        for (int u = u0; u < u1; ++u) {
+            float* p = row + (int64_t)u * d;
+            const float* bias = u < H ? (qb ? qb + (int64_t)u * d : nullptr) : (kb ? kb + (int64_t)(u - H) * d : nullptr);
+            const float x0 = bias ? p[a] + bias[a] : p[a], x1 = bias ? p[b] + bias[b] : p[b];
+            const float r0 = x0 * cs - x1 * sn, r1 = x1 * cs + x0 * sn;
+            if (u < H) {
+                p[a] = r0;
+                p[b] = r1;
+            } else if (slot >= 0) {
+                T_* kdst = kc + (slot + (u - H)) * d;
+                T_* vdst = vc + (slot + (u - H)) * d;
+                ActS<F32>::st(kdst + a, r0);
+                ActS<F32>::st(kdst + b, r1);
+                ActS<F32>::st(vdst + a, x0);
+                ActS<F32>::st(vdst + b, x1);
+            }
         }
     }
-    for (int c = rot + lane; c < d; c += 64) {
-        const float x0 = bias ? p[c] + bias[c] : p[c];
-        if (u < H) {
-            p[c] = x0;
-        } else {
-            ActS<F32>::st(kdst + c, x0);
-            ActS<F32>::st(vdst + c, x0);
+    for (int u = u0; u < u1; ++u) {
+        float* p = row + (int64_t)u * d;
+        const float* bias = u < H ? (qb ? qb + (int64_t)u * d : nullptr) : (kb ? kb + (int64_t)(u - H) * d : nullptr);
+        for (int c = rot + lane; c < d; c += 64) {
+            const float x0 = bias ? p[c] + bias[c] : p[c];
+            if (u < H) {
+                p[c] = x0;
+            } else if (slot >= 0) {
+                ActS<F32>::st(kc + (slot + (u - H)) * d + c, x0);
+                ActS<F32>::st(vc + (slot + (u - H)) * d + c, x0);
+            }
         }
     }
 }
@@ -1521,13 +1526,15 @@ int mv_qk_rotary_store(float* qk, int64_t ld, const float* q_bias, const float* 
         ld < (int64_t)(heads + kv_heads) * d)
         return MV_ERR_INVALID_ARG;
     PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
-    const int64_t units = (int64_t)tokens * (heads + kv_heads);
+    // steps of many tokens: a wave takes eight heads of a token and forms the angles' sines and cosines once for them
+    const int hpw = (int64_t)tokens * (heads + kv_heads) >= 8 * 1024 ? 8 : 1;
+    const int64_t units = (int64_t)tokens * ((heads + kv_heads + hpw - 1) / hpw);
     const int64_t rot_blocks = (units + 3) / 4, act_blocks = act_in ? (int64_t)tokens * ((act_n + 255) / 256) : 0;
     if (rot_blocks + act_blocks > 0x7fffffff) return MV_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)(rot_blocks + act_blocks));
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(qk_rotary_store_kernel<true>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
-    else hipLaunchKernelGGL(qk_rotary_store_kernel<false>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
+    if (f32) hipLaunchKernelGGL(qk_rotary_store_kernel<true>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, hpw, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
+    else hipLaunchKernelGGL(qk_rotary_store_kernel<false>, grid, dim3(256), 0, s, qk, ld, q_bias, k_bias, k_cache, v_cache, inv_freq, pr, tokens, heads, kv_heads, d, rot, adjacent, hpw, (unsigned)rot_blocks, act_in, lda, act_out, ldao, act_n, act_kind, act_limit, act_slope);
     return check_launch();
 }
 

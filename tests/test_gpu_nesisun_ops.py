@@ -398,6 +398,36 @@ def test_values_are_the_keys_before_rotation(ops):
         assert (q2 - qw).abs().max().item() < 1e-5
 
 
+@pytest.mark.parametrize("f32", [True, False])
+def test_rotation_over_a_step_of_many_tokens(ops, f32):
+    """Steps of many tokens form a position's sines and cosines once for several heads (a wave takes eight of them, a
+    last group of fewer): queries in place, keys and values in their pages, all as head by head."""
+    H, G, d, rot, base = 9, 3, 40, 24, 5000.0          # twelve heads: a group of eight and one of four
+    dt = torch.float32 if f32 else torch.bfloat16
+    g = torch.Generator().manual_seed(9)
+    T = 700
+    qk, qb, kb = attn_case(g, T, H, G, d)
+    cache = make_cache(kv={0: (G, d, d)}, dtype=dt, max_tokens=1024)
+    cache.k_caches[0].fill_(7.0)
+    parts = []
+    for lo, hi in ((0, 690), (690, 700)):              # the long step, then a short one (a wave per head) behind it
+        st = step_of(cache, [("r", [0] * (hi - lo))])
+        inv = (base ** (-2.0 * torch.arange(rot // 2, dtype=torch.float64) / rot)).to(DEV)
+        x = qk[lo:hi].to(DEV).clone()
+        ops.qk_rotary_store(x, qb.to(DEV), kb.to(DEV), cache.k_caches[0], cache.v_caches[0], inv, st, H, G, d, rot)
+        parts.append(x[:, :H * d].cpu().double())
+    pos = torch.arange(T)
+    k = (qk[:, H * d:].double() + kb.double()).view(T, G, d)
+    q = (qk[:, :H * d].double() + qb.double()).view(T, H, d)
+    pages = cache.get_blocks("r")
+    vals = torch.cat([cache.v_caches[0][p] for p in pages])[:T].float().cpu().double()
+    keys = torch.cat([cache.k_caches[0][p] for p in pages])[:T].float().cpu().double()
+    tol = 1e-5 if f32 else 3e-2
+    assert (torch.cat(parts).view(T, H, d) - ref.rotate_adjacent(q, pos, rot, base)).abs().max().item() < 1e-5
+    assert (keys - ref.rotate_adjacent(k, pos, rot, base)).abs().max().item() < tol
+    assert (vals - k).abs().max().item() < tol
+
+
 # ---------------------------------------------------------------------------------------------------- experts
 @pytest.mark.parametrize("f32", [False, True])
 @pytest.mark.parametrize("E,n_id,top", [(5, 2, 3), (4, 0, 1), (1, 1, 2), (12, 3, 4), (40, 1, 6), (2, 4, 2)])
