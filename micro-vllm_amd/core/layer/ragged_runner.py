@@ -443,10 +443,13 @@ class RaggedRunner:
         qk = proj[:, :(H + G) * d]
         kc, vc = cache.k_caches[li], cache.v_caches[li]
         cat = self._actbuf(T, H * d + ff)                          # [attention output | activations]
-        # gelu_tanh(gate) * up lands next to where the attention output will go, out of the rotation's launch
+        # gelu_tanh(gate) * up lands next to where the attention output will go.  In steps of few tokens it comes out of
+        # the rotation's launch (a launch saved); in long ones it runs behind the attention, whose keys and values the
+        # activations' traffic would otherwise push out of the caches
+        act = (proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH, 0.0, 1.0) if dense else None
+        fuse_act = dense and T <= 64
         ops.qk_rotary_store(qk, w["q_b"], w["k_b"], kc, vc, w["inv_freq"], step, H, G, d, int(m["rot"]["dims"]),
-                            adjacent=True,
-                            act=(proj[:, (H + G) * d:], cat[:, H * d:], ops.GATE_GELU_TANH, 0.0, 1.0) if dense else None)
+                            adjacent=True, act=act if fuse_act else None)
         window, keep = int(m["mask"]["size"]), int(m["mask"].get("keep_first", 0))
         # tokens of short rows (decoding): the query heads of a key/value head share its reads, the keys are cut over
         # several workgroups and the pieces meet in `part`
@@ -454,6 +457,8 @@ class RaggedRunner:
         part = self._f32buf(1, T * H * splits * (d + 2)) if splits else None
         ops.window_attn(qk, kc, vc, cat[:, :H * d], step, None, H, G, d, d, float(m["scale"]), window,
                         tiled=self.tiled_attn, keep_first=keep, sinks=w["sink"], part=part, splits=splits)
+        if dense and not fuse_act:
+            ops.gated_act(act[0], act[1], act[2])
         y1 = w["w_out"](cat, self._f32buf(T, self.width))
         if not mlp or dense:
             return y1, None
