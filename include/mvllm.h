@@ -698,6 +698,7 @@ int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place
                 mv_stream_t stream);
 /* s_t = sum_k weights[t,k] * expert_out[place[t*top+k]] (+ shared_gate[t] * shared_out[t]).  norm_w == NULL: y = s.
  * Else y is the residual stream: y += tanh(norm_alpha s) norm_w + norm_b, and h (optional) = act(y).
+ * weights == NULL: every weight is one; shared_gate == NULL: the shared expert's output counts whole.
  * ids != NULL: a choice ids[t*top+k] >= first_pass has no expert row; it adds weights[t,k] * pass[t,:] (activation
  * type, row stride ldp): an expert that hands its input through. */
 int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
@@ -705,6 +706,59 @@ int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, c
                    const float* norm_w, const float* norm_b, const float* norm_alpha, void* h, int64_t ldh, int tokens,
                    int n, int top, int f32, const int32_t* ids, int first_pass, const void* pass, int64_t ldp,
                    mv_stream_t stream);
+
+/* The `top` largest of W_router h (fp32; ties to the lower index); weights = sigmoid of each chosen output, not
+ * renormalised. */
+int mv_moe_route_sigmoid(const void* h, int64_t ldh, const float* w_router, int32_t* ids, float* weights, int tokens,
+                         int n, int experts, int top, int f32, mv_stream_t stream);
+/* mv_gated_act on rows sorted by expert, with both halves scaled first: out = act( f(s a[:, :n]) * (s a[:, n:2n]) ),
+ * s = scale[order[row]] (order == NULL: scale[row]): an expert that reads weight * h, from the products of h. */
+int mv_gated_act_scaled(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int kind, float limit,
+                        float slope, const float* scale, const int32_t* order, int f32, mv_stream_t stream);
+
+/* ---- gated residual stream, loop input (stream_ops.hip) ------------------------------------------------- */
+
+/* mode 1: x += y * sigmoid(g + b) (b == NULL: no bias); mode 2: x = y + b; mode 0: x as it is.  w != NULL:
+ * n = x / sqrt(mean(x^2) + eps) * (offset + w) of the new x, to n32 (fp32) and / or h (activation type). */
+int mv_gated_residual_norm(const float* y, int64_t ldy, const float* g, int64_t ldg, const float* b, int mode, float* x,
+                           int64_t ldx, const float* w, float eps, float offset, float* n32, int64_t ldn, void* h,
+                           int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
+/* out[r, :n] = act(a[r, :]), out[r, n:2n] = act(b[r, :]). */
+int mv_cast_concat(const float* a, int64_t lda, const float* b, int64_t ldb, void* out, int64_t ldo, int rows, int n,
+                   int f32, mv_stream_t stream);
+/* out = act( gelu(in) ), the tanh form. */
+int mv_gelu_tanh(const float* in, int64_t ldi, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+/* v[i] *= factor. */
+int mv_scale(float* v, int64_t count, float factor, mv_stream_t stream);
+
+/* ---- short convolutions without activation, differential attention (seq_mix.hip, diff_attn.hip) ---------- */
+
+/* y_t = (add_input ? u_t : 0) + sum_j w[c, j] u_(t - taps + 1 + j) per channel over a ragged step, inputs before
+ * the step from state [slots, taps - 1, channels] (zeros for a row with row_ctx == 0); y to out32 (fp32) and / or
+ * out_act (activation type); then the state keeps each row's last taps - 1 inputs. */
+int mv_conv_taps(const float* in, int64_t ldi, float* state, const float* w, float* out32, int64_t ld32, void* out_act,
+                 int64_t ldoa, int add_input, const int32_t* tok_row, const int32_t* row_start, const int32_t* row_len,
+                 const int32_t* row_ctx, const int32_t* row_slot, int tokens, int rows, int channels, int taps, int f32,
+                 mv_stream_t stream);
+/* The same convolution (taps == 0: none) over the cq + ck + cv columns of one projection: the first cq to q (fp32),
+ * the next ck into the token's row of k_cache [pages, page, ck], the last cv into v_cache [pages, page, cv]. */
+int mv_conv_qkv_store(const float* in, int64_t ldi, float* state, const float* w, float* q, int64_t ldq, void* k_cache,
+                      void* v_cache, const int32_t* tok_row, const int32_t* tok_pos, const int32_t* row_start,
+                      const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot,
+                      const int32_t* block_table, int bt_stride, int page, int tokens, int rows, int cq, int ck, int cv,
+                      int taps, int f32, mv_stream_t stream);
+/* Two causal softmax maps per head over the same values: q [T, heads, 2, d] fp32, k_cache [pages, page, kv_heads, 2, d],
+ * v_cache [pages, page, kv_heads, dv]; score = q.k * scale, then cap * tanh(score / cap) when cap > 0;
+ * o = a1 - lambda a2; out[t, h, :] = act( o / sqrt(mean(o^2) + eps) * out_scale * sigmoid(gate[t, h]) ) (gate == NULL:
+ * no gate).  chunks > 0: rows of more than max_len tokens run on the matrix cores where the shape allows it (bf16,
+ * pages of 64, (d, dv) in {(32,32), (32,64), (64,64), (64,128), (128,128)}); short_tokens = tokens in the other rows
+ * (-1: unknown). */
+int mv_diff_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
+                 const float* gate, int64_t ldg, const int32_t* tok_row, const int32_t* tok_pos,
+                 const int32_t* block_table, int bt_stride, int page, int tokens, int heads, int kv_heads, int d, int dv,
+                 float scale, float cap, float lambda, float out_scale, float eps, int f32, const int32_t* row_len,
+                 const int32_t* ch_start, const int32_t* ch_len, int chunks, int max_len, int short_tokens,
+                 mv_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -138,6 +138,17 @@ PROTOTYPES = {
     "mv_moe_plan": (_I, [_P, _P, _P, _P, _I, _I, _P]),
     "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P, _I, _P, _L,
                             _P]),
+    "mv_moe_route_sigmoid": (_I, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mv_gated_act_scaled": (_I, [_P, _L, _P, _L, _I, _I, _I, _F, _F, _P, _P, _I, _P]),
+    "mv_gated_residual_norm": (_I, [_P, _L, _P, _L, _P, _I, _P, _L, _P, _F, _F, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_cast_concat": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_gelu_tanh": (_I, [_P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_scale": (_I, [_P, _L, _F, _P]),
+    "mv_conv_taps": (_I, [_P, _L, _P, _P, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mv_conv_qkv_store": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                               _I, _I, _I, _P]),
+    "mv_diff_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _F, _F,
+                          _I, _P, _P, _P, _I, _I, _I, _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),

@@ -31,6 +31,7 @@ SOURCES = [
     "seq_mix.hip",
     "latent_attn.hip",
     "moe.hip",
+    "diff_attn.hip",
 ]
 
 # Libraries that hold a part of the sources, `lib/libmvllm_<name>.so`: what one model family needs, for a
@@ -40,7 +41,7 @@ SETS = {
     # fp32 residual stream, recurrent mixers, windowed attention; the wave-tile projections for the
     # shapes they take, and the sampler
     "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "latent_attn.hip", "moe.hip",
-               "elementwise.hip", "wgemm.hip", "gemm_prefill.hip", "sampler.hip"],
+               "diff_attn.hip", "elementwise.hip", "wgemm.hip", "gemm_prefill.hip", "sampler.hip"],
 }
 
 # -ffp-contract=off: rounding is part of the parity contract; FMAs are written explicitly
@@ -70,6 +71,7 @@ FILE_FLAGS = {
     "seq_mix.hip": _NO_PACKED_F32,
     "latent_attn.hip": _NO_PACKED_F32,
     "moe.hip": _NO_PACKED_F32,
+    "diff_attn.hip": _NO_PACKED_F32,
 }
 
 

@@ -49,8 +49,25 @@ Per layer (Nesisun; both sublayers of a layer read ONE RMS norm and enter the st
             sorted by expert -> gate|up by segment -> clamped gate -> down by segment -> weighted sum, a choice of
             a pass-through expert adding h itself; W_o separately
   then      x += both, and the NEXT layer's norm of the new x, in one launch
+
+Per layer (Solopel; pre-norm, every sublayer output passes a sigmoid gate computed from the sublayer's normed input):
+  residual  x += y * sigmoid(g + b) of the sublayer before, and the norm (weight 1 + w) of the new x, in one launch:
+            n in fp32 for the convolution and in the activation type for the gate projection R n
+  canon     act( n + conv(n) ): a short causal convolution per channel in front of the mixer, its last inputs kept per slot
+  latent attention  fused q|dkv projection -> the normed latent into the page, q in the activation type -> per-head
+            product carrying q into the latent space -> causal attention over the cached latents -> per-head value
+            up-projection -> cast -> out-projection
+  differential attention  fused q|k|v|gate projection -> short convolution over q|k|v (inputs kept per slot), keys and
+            values into the pages -> two softmax maps per head over the same values, their difference unit-normed and
+            gated per head, in one launch -> out-projection
+  dense     fused up|R2 projection -> gelu_tanh -> down
+  moe       router (fp32, sigmoid scores, top-k) -> pairs sorted by expert -> gate|up by segment -> SiLU-gate of the
+            products scaled by the pair's score (the score scales the expert's input) -> down by segment; shared
+            expert's gate|up|R2 in one projection; plain sum
+  loop      a pass of the looped span starts from W_in [x | x0] + step_t, x0 the embedding
 """
 import logging
+import math
 from typing import Dict, List, Optional
 
 import torch
@@ -90,6 +107,7 @@ class RaggedRunner:
         self.runs = cfg.layer_runs()
         self.sandwich = cfg.architecture == "Fagunex"     # Dynamic Tanh before and after each sublayer
         self.parallel_prenorm = cfg.architecture == "Nesisun"   # one RMS norm feeds mixer and feed-forward alike
+        self.gated_prenorm = cfg.architecture == "Solopel"      # pre-norm layers whose sublayer outputs pass a gate
         for wi, layer in self.runs:
             if wi not in self._w:
                 self._w[wi] = self._prepare_layer(wi, layer)
@@ -100,9 +118,15 @@ class RaggedRunner:
         elif self.parallel_prenorm:
             self.final_norm = self._small(model.get("final.norm"))
             self.pair_embed = self._act(model.get("bigram"))
+        elif self.gated_prenorm:
+            self.final_norm = self._small(model.get("final.norm"))
+            if cfg.loop:
+                self.loop_in = self._linear(model.get("loop.in"))
+                self.loop_step = self._small(model.get("loop.step"))
         else:
             self.final_norm = self._small(model.get("final.norm"))
-        self.head = self._linear(model.get("head"))
+        # Solopel's output head is its embedding table
+        self.head = self._linear(model.get("embed" if self.gated_prenorm else "head"))
 
     # ------------------------------------------------------------------ weights
     def _act(self, t):
@@ -132,6 +156,8 @@ class RaggedRunner:
             return self._prepare_fagunex(i, layer)
         if self.parallel_prenorm:
             return self._prepare_nesisun(i, layer)
+        if self.gated_prenorm:
+            return self._prepare_solopel(i, layer)
         g, p, m = self.model.get, f"l{i}.", layer["mixer"]
         w = {"norm1": self._small(g(p + "norm1"))}
         if layer["type"] == "mamba2":
@@ -223,10 +249,69 @@ class RaggedRunner:
                          e_down=self._stacked([g(p + f"mlp.e{e}.down") for e in range(E)]))
         return w
 
+    def _prepare_solopel(self, i: int, layer: dict) -> dict:
+        g, p, m, cfg, W = self.model.get, f"l{i}.", layer["mixer"], self.cfg, self.width
+        w = {"norm1": self._small(g(p + "norm1")), "rg1": self._linear(g(p + "rg1")), "rg1_b": self._small(g(p + "rg1.b"))}
+        if cfg.taps:
+            w["canon"] = self._small(g(p + "canon1"))
+        H, d, dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        if layer["type"] == "latent_attention":
+            R = int(m["kv_rank"])
+            # per head: q_abs = W_uk,h^T q (so the stacked weight is [H, R, d]), value = W_uv,h * latent sum ([H, dv, R])
+            uk = g(p + "mix.uk").reshape(H, d, R).transpose(1, 2)
+            uv = g(p + "mix.uv").reshape(H, dv, R)
+            w.update(w_in=self._linear(g(p + "mix.q"), g(p + "mix.dkv")), kv_norm=self._small(g(p + "mix.dkv.norm")),
+                     uk_t=self._stacked(list(uk)), uv=self._stacked(list(uv)), w_o=self._linear(g(p + "mix.o")))
+        else:
+            G, taps = int(m["kv_heads"]), int(m.get("conv") or 0)
+            C = H * 2 * d + G * 2 * d + G * dv
+            # the per-head gate rides the q | k | v projection; zero rows fill its width up to what the wave-tile
+            # projections take
+            pad = (-(C + H)) % 16
+            parts = [g(p + "mix.q"), g(p + "mix.k"), g(p + "mix.v"), g(p + "mix.g")]
+            if pad:
+                parts.append(torch.zeros(pad, W, dtype=parts[0].dtype))
+            dot = lambda a, b: float((g(p + a).double() * g(p + b).double()).sum())   # noqa: E731
+            diff = float(m["diff"])
+            w.update(w_in=self._linear(*parts), w_o=self._linear(g(p + "mix.o")),
+                     lam=math.exp(dot("mix.lq1", "mix.lk1")) - math.exp(dot("mix.lq2", "mix.lk2")) + diff,
+                     conv=self._small(torch.cat([g(p + "mix.q.conv"), g(p + "mix.k.conv"), g(p + "mix.v.conv")], dim=0))
+                     if taps else None)
+        mlp = layer.get("mlp")
+        if mlp:
+            w.update(norm2=self._small(g(p + "norm2")), rg2_b=self._small(g(p + "rg2.b")))
+            if mlp["kind"] == "dense":
+                # the feed-forward and its output gate read the same normed vector: one projection
+                w.update(up_rg=self._linear(g(p + "mlp.up"), g(p + "rg2")), down=self._linear(g(p + "mlp.down")))
+            else:
+                E = int(mlp["router"]["experts"])
+                w.update(router=self._small(g(p + "mlp.router")),
+                         e_gu=self._stacked([torch.cat([g(p + f"mlp.e{e}.gate"), g(p + f"mlp.e{e}.up")], dim=0)
+                                             for e in range(E)]),
+                         e_down=self._stacked([g(p + f"mlp.e{e}.down") for e in range(E)]))
+                if mlp.get("shared"):
+                    w.update(s_gu_rg=self._linear(g(p + "mlp.shared.gate"), g(p + "mlp.shared.up"), g(p + "rg2")),
+                             s_down=self._linear(g(p + "mlp.shared.down")))
+                else:
+                    w.update(rg2=self._linear(g(p + "rg2")))
+        return w
+
     # ------------------------------------------------------------------ cache geometry
     def cache_layout(self):
         """(kv_layers, state_layers) for HybridCacheManager: what every layer RUN keeps per sequence."""
         kv, state = {}, {}
+        if self.gated_prenorm:
+            for i, (_, layer) in enumerate(self.runs):
+                m = layer["mixer"]
+                state[i] = {"canon": (self.cfg.taps - 1, self.width)} if self.cfg.taps else {}
+                if layer["type"] == "latent_attention":
+                    kv[i] = (1, int(m["kv_rank"]), 0)          # one normed latent per token: key and value alike
+                else:
+                    H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+                    kv[i] = (G, 2 * d, dv)                     # both maps' keys of a key/value head side by side
+                    if int(m.get("conv") or 0) > 1:
+                        state[i]["qkv"] = (int(m["conv"]) - 1, H * 2 * d + G * 2 * d + G * dv)
+            return kv, state
         for i, (_, layer) in enumerate(self.runs):
             m = layer["mixer"]
             if layer["type"] == "mamba2":
@@ -392,6 +477,8 @@ class RaggedRunner:
                 ops.add_rmsnorm(x, y1, y2, w=nxt, eps=cfg.eps, h=None if nxt is None else h)
                 if residuals is not None:
                     residuals.append(x.clone())
+        elif self.gated_prenorm:
+            x = self._solopel_stack(step, cache, residuals)
         elif self.sandwich:
             ops.embed_scaled(self.embed, step.ids, 1.0, x, h)
             for li, (wi, layer) in enumerate(self.runs):
@@ -427,6 +514,8 @@ class RaggedRunner:
         else:
             ops.offset_rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
         logits = self.head(normed, self._f32buf(rows, self.vocab_size))
+        if getattr(cfg, "logit_scale", 1.0) != 1.0:
+            ops.scale_(logits, cfg.logit_scale)
         if getattr(cfg, "logit_softcap", None):
             ops.softcap_(logits, cfg.logit_softcap)
         return logits
@@ -481,6 +570,117 @@ class RaggedRunner:
         y = self._f32buf(T, self.width)
         ops.moe_combine(down, place, wts, None, None, y, ids=ids.view(-1), first_pass=E, passed=h)
         return y
+
+    # ------------------------------------------------------------------ Solopel layers
+    def _solopel_stack(self, step: RaggedStep, cache: HybridCacheManager, residuals):
+        """All layer runs on a fresh stream; returns it.  A sublayer's output enters the stream in the launch that
+        forms the NEXT norm, so between layers it travels as `pend` = (y, gate logits, gate bias, replace)."""
+        cfg, T, W = self.cfg, step.tokens, self.width
+        plan = cfg.run_plan()
+        x0, x, h = self._f32buf(T, W), self._f32buf(T, W), self._actbuf(T, W)
+        ops.embed_scaled(self.embed, step.ids, 1.0, x0, h)
+        if plan[0][1] < 0:
+            ops.embed_scaled(self.embed, step.ids, 1.0, x, h)
+        pend = None
+        for li, ((wi, layer), (_, t_pass)) in enumerate(zip(self.runs, plan)):
+            if t_pass >= 0:       # a pass of the looped span starts: x = W_in [x | x0] + step_t
+                if pend is not None:
+                    ops.gated_residual_norm(x, *pend)
+                cat = self._actbuf(T, 2 * W)
+                ops.cast_concat(x if li > 0 else x0, x0, cat)
+                pend = (self.loop_in(cat, self._f32buf(T, W)), None, self.loop_step[t_pass], True)
+            pend = self._solopel_layer(li, self._w[wi], layer, x, pend, step, cache)
+            if residuals is not None:
+                ops.gated_residual_norm(x, *pend)
+                pend = None
+                residuals.append(x.clone())
+        if pend is not None:
+            ops.gated_residual_norm(x, *pend)
+        return x
+
+    def _solopel_layer(self, li, w, layer, x, pend, step: RaggedStep, cache: HybridCacheManager):
+        T, W, cfg, eps = step.tokens, self.width, self.cfg, self.cfg.eps
+        y, g, b, replace = pend if pend is not None else (None, None, None, False)
+        h = self._actbuf(T, W)
+        # the convolution reads the norm in fp32; in fp32 runs that is h itself
+        n32 = self._f32buf(T, W) if cfg.taps and self.dtype != torch.float32 else None
+        ops.gated_residual_norm(x, y, g, b, replace, w=w["norm1"], eps=eps, offset=1.0, n32=n32, h=h)
+        hc = h
+        if cfg.taps:
+            hc = self._actbuf(T, W)
+            ops.conv_taps(h if n32 is None else n32, cache.states[li]["canon"], w["canon"], step, out_act=hc,
+                          add_input=True)
+        g1 = w["rg1"](h, self._f32buf(T, W))
+        if layer["type"] == "latent_attention":
+            y = self._solopel_latent(li, w, layer["mixer"], hc, step, cache)
+        else:
+            y = self._solopel_diff(li, w, layer["mixer"], hc, step, cache)
+        mlp = layer.get("mlp")
+        if not mlp:
+            return y, g1, w["rg1_b"], False
+        h2 = self._actbuf(T, W)
+        ops.gated_residual_norm(x, y, g1, w["rg1_b"], w=w["norm2"], eps=eps, offset=1.0, h=h2)
+        if mlp["kind"] == "dense":
+            ff = int(mlp["ff"])
+            proj = w["up_rg"](h2, self._f32buf(T, ff + W))            # [up | gate logits of the residual]
+            act = self._actbuf(T, ff)
+            ops.gelu_tanh(proj[:, :ff], act)
+            return w["down"](act, self._f32buf(T, W)), proj[:, ff:], w["rg2_b"], False
+        E, top, ff = int(mlp["router"]["experts"]), int(mlp["router"]["top"]), int(mlp["expert"]["ff"])
+        ids = self._i32buf(T * top).view(T, top)
+        wts = self._f32buf(T, top)
+        ops.moe_route_sigmoid(h2, w["router"], ids, wts)
+        seg, order, place = self._i32buf(E + 1), self._i32buf(T * top), self._i32buf(T * top)
+        ops.moe_plan(ids, seg, order, place, E)
+        # an expert reads score * h: its gate and up products are linear in h, so the score goes onto the products
+        gu = ops.linear_segments(h2, w["e_gu"], self._f32buf(T * top, 2 * ff), seg, order, top, T)
+        act = self._actbuf(T * top, ff)
+        ops.gated_act_scaled(gu, act, ops.GATE_SILU, wts.view(-1), order)
+        down = ops.linear_segments(act, w["e_down"], self._f32buf(T * top, W), seg, None, 1, T)
+        s_out = None
+        if mlp.get("shared"):
+            sf = int(mlp["shared"]["ff"])
+            proj = w["s_gu_rg"](h2, self._f32buf(T, 2 * sf + W))     # [gate | up | gate logits of the residual]
+            s_act = self._actbuf(T, sf)
+            ops.silu_mul(proj[:, :2 * sf], s_act)
+            s_out, g2 = w["s_down"](s_act, self._f32buf(T, W)), proj[:, 2 * sf:]
+        else:
+            g2 = w["rg2"](h2, self._f32buf(T, W))
+        y2 = self._f32buf(T, W)
+        ops.moe_combine(down, place, None, s_out, None, y2)
+        return y2, g2, w["rg2_b"], False
+
+    def _solopel_latent(self, li, w, m, hc, step: RaggedStep, cache: HybridCacheManager):
+        T, eps = step.tokens, self.cfg.eps
+        H, d, dv, R = int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"])
+        proj = w["w_in"](hc, self._f32buf(T, H * d + R))               # [q | dkv]
+        pages = cache.k_caches[li]
+        pages = pages.view(pages.shape[0], pages.shape[1], R)
+        q_plain, q_abs = self._actbuf(T, H * d), self._f32buf(T, H * R)
+        ops.latent_prep(proj[:, H * d:], w["kv_norm"], eps, pages, proj[:, :H * d], q_plain, q_abs, None, step, H, d, 0,
+                        R, 0, interleaved=False)
+        ops.linear_heads(q_plain, w["uk_t"], q_abs.view(T, H, R), H)
+        lat = self._actbuf(T, H * R)
+        ops.latent_attn(q_abs, pages, lat, step, None, H, R, 0, float(m["scale"]), 0, tiled=self.tiled_attn)
+        val = self._f32buf(T, H * dv)
+        ops.linear_heads(lat, w["uv"], val.view(T, H, dv), H)
+        a = self._actbuf(T, H * dv)
+        ops.sigmoid_gate(val, None, a)
+        return w["w_o"](a, self._f32buf(T, self.width))
+
+    def _solopel_diff(self, li, w, m, hc, step: RaggedStep, cache: HybridCacheManager):
+        T = step.tokens
+        H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+        C = H * 2 * d + G * 2 * d + G * dv
+        proj = w["w_in"](hc, self._f32buf(T, w["w_in"].n))             # [q | k | v | head gates (| zeros)]
+        q = self._f32buf(T, H * 2 * d)
+        kc, vc = cache.k_caches[li], cache.v_caches[li]
+        ops.conv_qkv_store(proj, cache.states[li].get("qkv"), w["conv"], q, kc, vc, step)
+        a = self._actbuf(T, H * dv)
+        diff = float(m["diff"])
+        ops.diff_attn(q, kc, vc, a, proj[:, C:C + H], step, H, G, d, dv, float(m["scale"]), float(m.get("softcap") or 0.0),
+                      w["lam"], 1.0 - diff, self.cfg.eps, tiled=self.tiled_attn)
+        return w["w_o"](a, self._f32buf(T, self.width))
 
     # ------------------------------------------------------------------ Fagunex layers
     def _i32buf(self, count):

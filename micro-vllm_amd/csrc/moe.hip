@@ -8,6 +8,11 @@
 //                score + correction are chosen (ties: the lower index), their weights are the scores themselves
 //                (without the correction) divided by their sum (+ floor), times `scale`.  Router outputs from
 //                `first_pass` on have no expert behind them: they stand for the input itself (moe_combine)
+//   moe_route_sigmoid  the `top` largest fp32 logits (ties: the lower index), weights = sigmoid of each chosen
+//                logit, not renormalised
+//   gated_act_scaled  rows sorted by expert: out = act( f(s g) * (s u) ) with s the weight of the row's (token,
+//                choice) pair - an expert that reads weight * h, formed from the products of h itself (the
+//                projections are linear)
 //   moe_plan     the step's T * top (token, choice) pairs sorted by expert: seg[e] .. seg[e+1] are expert e's
 //                rows, order[i] the pair (token * top + choice) in row i, place[pair] its row.  The order inside
 //                an expert is whatever the atomics give; no result depends on it, since a row's products do
@@ -25,7 +30,7 @@ constexpr int kMaxExperts = 1024, kMaxTop = 16;
 template <bool F32>
 __global__ __launch_bounds__(256) void moe_route_kernel(const void* h_, int64_t ldh, const float* wr, const float* wsg,
                                                         int* ids, float* wts, float* shared_gate, int n, int E,
-                                                        int top) {
+                                                        int top, int sigmoid_scores) {
     __shared__ float z[kMaxExperts + 1];
     const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int units = E + (wsg ? 1 : 0);
@@ -65,9 +70,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const void* h_, int64_t 
         float sum = 0.f;
         const float largest = val[0];
         for (int k = 0; k < top; ++k) {
-            val[k] = expf(val[k] - largest);
+            val[k] = sigmoid_scores ? 1.0f / (1.0f + expf(-val[k])) : expf(val[k] - largest);
             sum += val[k];
         }
+        if (sigmoid_scores) sum = 1.0f;      // each chosen expert keeps its own score
         for (int k = 0; k < top; ++k) {
             ids[(int64_t)t * top + k] = pick[k];
             wts[(int64_t)t * top + k] = val[k] / sum;
@@ -172,10 +178,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64
     float w[kMaxTop];
     for (int k = 0; k < top; ++k) {
         rows[k] = place[(int64_t)t * top + k];
-        w[k] = wts[(int64_t)t * top + k];
+        w[k] = wts ? wts[(int64_t)t * top + k] : 1.0f;
         if (ids && ids[(int64_t)t * top + k] >= first_pass) rows[k] = -1;   // the input itself, not an expert's row
     }
-    const float g = so ? shared_gate[t] : 0.f;
+    const float g = so ? (shared_gate ? shared_gate[t] : 1.0f) : 0.f;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c < n) {
         float acc = 0.f;
@@ -198,6 +204,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64
     }
 }
 
+template <bool F32>
+__global__ __launch_bounds__(256) void gated_act_scaled_kernel(const float* a, int64_t lda, void* out_, int64_t ldo,
+                                                               int n, int kind, float limit, float slope,
+                                                               const float* scale, const int* order) {
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= n) return;
+    const float sc = scale[order ? order[row] : row];
+    const float v = gated_act_f(sc * a[row * lda + c], sc * a[row * lda + n + c], kind, limit, slope);
+    if (F32) ((float*)out_)[row * ldo + c] = v;
+    else ((uint16_t*)out_)[row * ldo + c] = (uint16_t)f32_to_bf16_bits(v);
+}
+
 }  // namespace mv
 
 extern "C" {
@@ -211,8 +230,8 @@ int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float*
     if (tokens == 0) return MV_OK;
     if (!h || !w_router || !ids || !weights || (w_shared_gate && !shared_gate) || ldh < n) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(moe_route_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top);
-    else hipLaunchKernelGGL(moe_route_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top);
+    if (f32) hipLaunchKernelGGL(moe_route_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top, 0);
+    else hipLaunchKernelGGL(moe_route_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top, 0);
     return check_launch();
 }
 
@@ -227,6 +246,32 @@ int mv_moe_route_scored(const void* h, int64_t ldh, const float* w_router, const
     hipStream_t s = (hipStream_t)stream;
     if (f32) hipLaunchKernelGGL(moe_route_scored_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, correction, ids, weights, n, experts, top, scale, sum_floor);
     else hipLaunchKernelGGL(moe_route_scored_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, correction, ids, weights, n, experts, top, scale, sum_floor);
+    return check_launch();
+}
+
+int mv_moe_route_sigmoid(const void* h, int64_t ldh, const float* w_router, int32_t* ids, float* weights, int tokens,
+                         int n, int experts, int top, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0 || experts <= 0 || experts > kMaxExperts || top <= 0 || top > kMaxTop || top > experts)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!h || !w_router || !ids || !weights || ldh < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(moe_route_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, (const float*)nullptr, ids, weights, (float*)nullptr, n, experts, top, 1);
+    else hipLaunchKernelGGL(moe_route_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, (const float*)nullptr, ids, weights, (float*)nullptr, n, experts, top, 1);
+    return check_launch();
+}
+
+int mv_gated_act_scaled(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int kind, float limit,
+                        float slope, const float* scale, const int32_t* order, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || kind < 0 || kind > 2) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !out || !scale || lda < 2 * (int64_t)n || ldo < n) return MV_ERR_INVALID_ARG;
+    const dim3 grid(rows, (n + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(gated_act_scaled_kernel<true>, grid, dim3(256), 0, s, a, lda, out, ldo, n, kind, limit, slope, scale, order);
+    else hipLaunchKernelGGL(gated_act_scaled_kernel<false>, grid, dim3(256), 0, s, a, lda, out, ldo, n, kind, limit, slope, scale, order);
     return check_launch();
 }
 
@@ -248,7 +293,7 @@ int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, c
     using namespace mv;
     if (tokens < 0 || n <= 0 || top <= 0 || top > kMaxTop) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
-    if (!expert_out || !place || !weights || !y || (shared_out && !shared_gate) || lde < n || ldy < n ||
+    if (!expert_out || !place || !y || lde < n || ldy < n ||
         (shared_out && lds < n))
         return MV_ERR_INVALID_ARG;
     if (norm_w ? (!norm_b || !norm_alpha || (h && ldh < n)) : h != nullptr) return MV_ERR_INVALID_ARG;

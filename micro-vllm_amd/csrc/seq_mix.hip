@@ -5,6 +5,10 @@
 // a row with row_ctx == 0 starts from zero state whatever its slot held before.
 //
 //   conv_silu / conv_state_update  short causal convolution per channel with its tail kept per slot
+//   conv_taps                      the same convolution without bias or activation, optionally added to its
+//                                  input (y = u + conv(u)); output in fp32 and / or the activation type
+//   conv_qkv_store                 the convolution over the q | k | v columns of one projection: queries to a
+//                                  buffer, keys and values straight into their pages
 //   softplus_decay                 step sizes and decays of a selective state-space head
 //   scan_outer                     S_t = decay_t S_(t-1) + gain_t k_t v_t^T,  o_t = S_t^T q_t (+ skip_h v_t)
 //                                  (state-space duality heads and fixed-decay retention heads alike)
@@ -684,6 +688,64 @@ __global__ __launch_bounds__(256) void qk_rotary_store_kernel(float* qk, int64_t
     }
 }
 
+// value of channel c at token t under a causal convolution of `taps` taps whose first inputs come from the slot
+__device__ __forceinline__ float conv_at(const float* in, int64_t ldi, const float* state, const float* w,
+                                         const StepRows& r, int t, int c, int C, int taps) {
+    const int b = r.tok_row[t];
+    const int rel = t - r.row_start[b];
+    const bool carried = r.row_ctx[b] > 0;
+    const float* st = state + ((int64_t)r.row_slot[b] * (taps - 1)) * C + c;
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int src = rel - (taps - 1) + j;
+        float v;
+        if (src >= 0) v = in[(int64_t)(t - (taps - 1) + j) * ldi + c];
+        else v = carried ? st[(int64_t)(src + taps - 1) * C] : 0.f;
+        acc = fmaf(w[(int64_t)c * taps + j], v, acc);
+    }
+    return acc;
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void conv_taps_kernel(const float* in, int64_t ldi, const float* state,
+                                                        const float* w, float* o32, int64_t ld32, void* oact_,
+                                                        int64_t ldoa, int add_input, StepRows r, int T, int C,
+                                                        int taps) {
+    typedef typename ActS<F32>::T T_;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)T * C) return;
+    const int t = (int)(i / C), c = (int)(i % C);
+    float v = conv_at(in, ldi, state, w, r, t, c, C, taps);
+    if (add_input) v += in[(int64_t)t * ldi + c];
+    if (o32) o32[(int64_t)t * ld32 + c] = v;
+    if (oact_) ActS<F32>::st((T_*)oact_ + (int64_t)t * ldoa + c, v);
+}
+
+// columns [0, Cq) -> q (fp32), [Cq, Cq + Ck) -> the token's row of the key page, the last Cv -> the value page.
+// w == NULL: no convolution, the columns go where they belong as they are
+template <bool F32>
+__global__ __launch_bounds__(256) void conv_qkv_store_kernel(const float* in, int64_t ldi, const float* state,
+                                                             const float* w, float* q, int64_t ldq, void* kc_,
+                                                             void* vc_, StepRows r, PagedRows pr, int T, int Cq,
+                                                             int Ck, int Cv, int taps) {
+    typedef typename ActS<F32>::T T_;
+    const int C = Cq + Ck + Cv;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)T * C) return;
+    const int t = (int)(i / C), c = (int)(i % C);
+    const float v = w ? conv_at(in, ldi, state, w, r, t, c, C, taps) : in[(int64_t)t * ldi + c];
+    if (c < Cq) {
+        q[(int64_t)t * ldq + c] = v;
+        return;
+    }
+    const int pos = pr.tok_pos[t];
+    const int pg = pr.block_table[(int64_t)pr.tok_row[t] * pr.bt_stride + pos / pr.page];
+    if (pg < 0) return;
+    const int64_t slot = (int64_t)pg * pr.page + pos % pr.page;
+    if (c < Cq + Ck) ActS<F32>::st((T_*)kc_ + slot * Ck + (c - Cq), v);
+    else ActS<F32>::st((T_*)vc_ + slot * Cv + (c - Cq - Ck), v);
+}
+
 constexpr int kMaxVC = 4;  // value columns per lane: vdim <= 256
 
 // One workgroup per (token, head).  Its NW waves (4, or 16 when a step has too few tokens to fill the
@@ -1307,6 +1369,59 @@ int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, con
         const int64_t w2 = (int64_t)rows * channels;
         hipLaunchKernelGGL(conv_state_update_kernel, dim3((unsigned)((w2 + 255) / 256)), dim3(256), 0, s, in, ldi, state,
                            r, rows, channels, taps);
+    }
+    return check_launch();
+}
+
+int mv_conv_taps(const float* in, int64_t ldi, float* state, const float* w, float* out32, int64_t ld32, void* out_act,
+                 int64_t ldoa, int add_input, const int32_t* tok_row, const int32_t* row_start, const int32_t* row_len,
+                 const int32_t* row_ctx, const int32_t* row_slot, int tokens, int rows, int channels, int taps, int f32,
+                 mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || rows < 0 || channels <= 0 || taps < 1 || taps > kMaxTaps) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!in || (!state && taps > 1) || !w || (!out32 && !out_act) || ldi < channels || (out32 && ld32 < channels) ||
+        (out_act && ldoa < channels) || !tok_row || !row_start || !row_len || !row_ctx || !row_slot)
+        return MV_ERR_INVALID_ARG;
+    StepRows r{tok_row, nullptr, row_start, row_len, row_ctx, row_slot};
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t work = (int64_t)tokens * channels;
+    const dim3 grid((unsigned)((work + 255) / 256));
+    if (f32) hipLaunchKernelGGL(conv_taps_kernel<true>, grid, dim3(256), 0, s, in, ldi, state, w, out32, ld32, out_act, ldoa, add_input, r, tokens, channels, taps);
+    else hipLaunchKernelGGL(conv_taps_kernel<false>, grid, dim3(256), 0, s, in, ldi, state, w, out32, ld32, out_act, ldoa, add_input, r, tokens, channels, taps);
+    if (taps > 1) {
+        const int64_t w2 = (int64_t)rows * channels;
+        hipLaunchKernelGGL(conv_state_update_kernel, dim3((unsigned)((w2 + 255) / 256)), dim3(256), 0, s, in, ldi, state,
+                           r, rows, channels, taps);
+    }
+    return check_launch();
+}
+
+int mv_conv_qkv_store(const float* in, int64_t ldi, float* state, const float* w, float* q, int64_t ldq, void* k_cache,
+                      void* v_cache, const int32_t* tok_row, const int32_t* tok_pos, const int32_t* row_start,
+                      const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot,
+                      const int32_t* block_table, int bt_stride, int page, int tokens, int rows, int cq, int ck, int cv,
+                      int taps, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || rows < 0 || cq <= 0 || ck <= 0 || cv <= 0 || taps < 0 || taps > kMaxTaps || page <= 0)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    const int C = cq + ck + cv;
+    if (!in || ldi < C || (taps > 0 && !w) || (taps > 1 && !state) || !q || ldq < cq || !k_cache || !v_cache ||
+        !tok_row || !tok_pos || !row_start || !row_len || !row_ctx || !row_slot || !block_table)
+        return MV_ERR_INVALID_ARG;
+    StepRows r{tok_row, tok_pos, row_start, row_len, row_ctx, row_slot};
+    PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t work = (int64_t)tokens * C;
+    const dim3 grid((unsigned)((work + 255) / 256));
+    const float* wk = taps > 0 ? w : nullptr;
+    if (f32) hipLaunchKernelGGL(conv_qkv_store_kernel<true>, grid, dim3(256), 0, s, in, ldi, state, wk, q, ldq, k_cache, v_cache, r, pr, tokens, cq, ck, cv, taps);
+    else hipLaunchKernelGGL(conv_qkv_store_kernel<false>, grid, dim3(256), 0, s, in, ldi, state, wk, q, ldq, k_cache, v_cache, r, pr, tokens, cq, ck, cv, taps);
+    if (taps > 1) {
+        const int64_t w2 = (int64_t)rows * C;
+        hipLaunchKernelGGL(conv_state_update_kernel, dim3((unsigned)((w2 + 255) / 256)), dim3(256), 0, s, in, ldi, state,
+                           r, rows, C, taps);
     }
     return check_launch();
 }

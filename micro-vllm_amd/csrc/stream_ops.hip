@@ -26,6 +26,13 @@
 //   rmsnorm_gather:      out = act( x[idx] / sqrt(mean(x[idx]^2) + eps) * (offset + w) )
 //   gated_act:           out = act( f(a[:, :n]) * a[:, n:2n] ), f = SiLU or the tanh form of GELU; or the clamped
 //                        gate  g' = min(g, limit), u' = clamp(u, +-limit): out = act( g' sigmoid(slope g') (u' + 1) )
+//   gated_residual_norm: the residual step of a pre-norm layer whose sublayer outputs pass a sigmoid gate:
+//                        x += y * sigmoid(g + b)  (mode 1), or  x = y + b  (mode 2: a new pass of a looped span
+//                        starts from a projection plus a per-pass vector); then n = x / sqrt(mean(x^2) + eps) *
+//                        (offset + w) as fp32 (what a convolution over time reads) and / or in the activation type
+//   cast_concat:         out = act( [a | b] )   (two fp32 streams side by side as one projection's operand)
+//   gelu_tanh:           out = act( gelu(in) ), the tanh form
+//   scale:               v *= s
 // All arithmetic is fp32 with the library's exact division, square root and tanh.
 #include "common.h"
 
@@ -334,6 +341,72 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const float* a, int64_t 
     Act<F32>::st(out + row * ldo + c, gated_act_f(a[row * lda + c], a[row * lda + n + c], kind, limit, slope));
 }
 
+
+// mode 0: x as it is; 1: x += y * sigmoid(g + b); 2: x = y + b.  w != NULL: the norm of the new x, to n32 (fp32)
+// and / or h (activation type)
+template <bool F32>
+__global__ __launch_bounds__(256) void gated_residual_norm_kernel(const float* y, int64_t ldy, const float* g,
+                                                                  int64_t ldg, const float* b, int mode, float* x,
+                                                                  int64_t ldx, const float* w, float eps, float offset,
+                                                                  float* n32, int64_t ldn, void* h_, int64_t ldh,
+                                                                  int n) {
+    typedef typename Act<F32>::T T;
+    __shared__ float red[4];
+    T* h = (T*)h_;
+    const int64_t row = blockIdx.x;
+    float* xr = x + row * ldx;
+    float ss = 0.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < n; c += 256) {
+        float v;
+        if (mode == 1) {
+            const float z = g[row * ldg + c] + (b ? b[c] : 0.f);
+            v = fmaf(y[row * ldy + c], 1.0f / (1.0f + expf(-z)), xr[c]);
+            xr[c] = v;
+        } else if (mode == 2) {
+            v = y[row * ldy + c] + (b ? b[c] : 0.f);
+            xr[c] = v;
+        } else {
+            v = xr[c];
+        }
+        ss += v * v;
+    }
+    if (!w) return;
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll 4
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float v = (xr[c] * inv) * (offset + w[c]);
+        if (n32) n32[row * ldn + c] = v;
+        if (h) Act<F32>::st(h + row * ldh + c, v);
+    }
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void cast_concat_kernel(const float* a, int64_t lda, const float* b, int64_t ldb,
+                                                          void* out_, int64_t ldo, int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= 2 * n) return;
+    Act<F32>::st(out + row * ldo + c, c < n ? a[row * lda + c] : b[row * ldb + (c - n)]);
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const float* in, int64_t ldi, void* out_, int64_t ldo, int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) Act<F32>::st(out + row * ldo + c, gelu_tanh_f(in[row * ldi + c]));
+}
+
+__global__ __launch_bounds__(256) void scale_kernel(float* v, int64_t count, float s) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) v[i] *= s;
+}
+
 }  // namespace mv
 
 extern "C" {
@@ -542,6 +615,56 @@ int mv_sigmoid_gate(const float* a, int64_t lda, const float* g, int64_t ldg, vo
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(rows, (n + 255) / 256);
     MV_F32_LAUNCH(sigmoid_gate_kernel, grid, a, lda, g, ldg, out, ldo, n);
+    return check_launch();
+}
+
+int mv_gated_residual_norm(const float* y, int64_t ldy, const float* g, int64_t ldg, const float* b, int mode, float* x,
+                           int64_t ldx, const float* w, float eps, float offset, float* n32, int64_t ldn, void* h,
+                           int64_t ldh, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || mode < 0 || mode > 2) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!x || ldx < n || (mode != 0 && (!y || ldy < n)) || (mode == 1 && (!g || ldg < n)) ||
+        (w && !n32 && !h) || (!w && (n32 || h)) || (n32 && ldn < n) || (h && ldh < n) || (!w && mode == 0))
+        return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(gated_residual_norm_kernel<true>, dim3(rows), dim3(256), 0, s, y, ldy, g, ldg, b, mode, x, ldx, w, eps, offset, n32, ldn, h, ldh, n);
+    else hipLaunchKernelGGL(gated_residual_norm_kernel<false>, dim3(rows), dim3(256), 0, s, y, ldy, g, ldg, b, mode, x, ldx, w, eps, offset, n32, ldn, h, ldh, n);
+    return check_launch();
+}
+
+int mv_cast_concat(const float* a, int64_t lda, const float* b, int64_t ldb, void* out, int64_t ldo, int rows, int n,
+                   int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !b || !out || lda < n || ldb < n || ldo < 2 * (int64_t)n) return MV_ERR_INVALID_ARG;
+    const dim3 grid(rows, (2 * n + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(cast_concat_kernel<true>, grid, dim3(256), 0, s, a, lda, b, ldb, out, ldo, n);
+    else hipLaunchKernelGGL(cast_concat_kernel<false>, grid, dim3(256), 0, s, a, lda, b, ldb, out, ldo, n);
+    return check_launch();
+}
+
+int mv_gelu_tanh(const float* in, int64_t ldi, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!in || !out || ldi < n || ldo < n) return MV_ERR_INVALID_ARG;
+    const dim3 grid(rows, (n + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(gelu_tanh_kernel<true>, grid, dim3(256), 0, s, in, ldi, out, ldo, n);
+    else hipLaunchKernelGGL(gelu_tanh_kernel<false>, grid, dim3(256), 0, s, in, ldi, out, ldo, n);
+    return check_launch();
+}
+
+int mv_scale(float* v, int64_t count, float factor, mv_stream_t stream) {
+    using namespace mv;
+    if (count < 0) return MV_ERR_INVALID_ARG;
+    if (count == 0) return MV_OK;
+    if (!v) return MV_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, (hipStream_t)stream, v, count,
+                       factor);
     return check_launch();
 }
 

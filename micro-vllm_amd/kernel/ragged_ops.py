@@ -499,22 +499,26 @@ def moe_plan(ids, seg, order, place, experts: int):
 
 def moe_combine(expert_out, place, weights, shared_out, shared_gate, y, norm=None, h=None, ids=None, first_pass: int = 0,
                 passed=None):
-    """y = the weighted sum of each token's experts (+ shared_gate * shared_out).  With `norm` y is the residual
+    """y = the weighted sum of each token's experts (+ shared_gate * shared_out; weights None: ones, shared_gate None:
+    one).  With `norm` y is the residual
     stream and receives the sum through that norm, y += tanh(alpha sum) w + b; h (optional) = y in the activation
     type.  With `ids` [tokens, top] a choice >= first_pass is an expert that hands its input through: it adds its
     weight times the token's row of `passed` (activation type)."""
     tokens, n = y.shape
-    top = weights.shape[1]
+    top = place.numel() // max(tokens, 1) if weights is None else weights.shape[1]
     assert ids is None or (ids.numel() == tokens * top and passed is not None and passed.shape == (tokens, n)
                            and passed.stride(1) == 1)
-    assert expert_out.shape == (tokens * top, n) and place.numel() == tokens * top and weights.is_contiguous()
-    assert shared_out is None or (shared_out.shape == (tokens, n) and shared_gate.numel() == tokens)
+    assert expert_out.shape == (tokens * top, n) and place.numel() == tokens * top
+    assert weights is None or (weights.shape == (tokens, top) and weights.is_contiguous())
+    assert shared_out is None or (shared_out.shape == (tokens, n) and (shared_gate is None or shared_gate.numel() == tokens))
     assert h is None or (norm is not None and h.shape == (tokens, n))
     w, b, a = _dyt(norm) if norm is not None else (None, None, None)
     nv.check("mv_moe_combine", nv.lib().mv_moe_combine(
-        _f32(expert_out).data_ptr(), _ld(expert_out), _i32(place).data_ptr(), _f32(weights).data_ptr(),
+        _f32(expert_out).data_ptr(), _ld(expert_out), _i32(place).data_ptr(),
+        None if weights is None else _f32(weights).data_ptr(),
         None if shared_out is None else _f32(shared_out).data_ptr(), 0 if shared_out is None else _ld(shared_out),
-        None if shared_out is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y), w, b, a,
+        None if shared_out is None or shared_gate is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y),
+        w, b, a,
         None if h is None else h.data_ptr(), 0 if h is None else _ld(h), tokens, n, top,
         _is_f32(passed) if passed is not None else (0 if h is None else _is_f32(h)),
         None if ids is None else _i32(ids).data_ptr(), int(first_pass), None if ids is None else passed.data_ptr(),
@@ -587,3 +591,140 @@ def rmsnorm_gather(x, idx, w, eps: float, out, offset: float = 0.0):
     nv.check("mv_rmsnorm_gather", nv.lib().mv_rmsnorm_gather(
         _f32(x).data_ptr(), _ld(x), None if idx is None else _i32(idx).data_ptr(), _f32(w).data_ptr(), float(eps),
         float(offset), out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Gated residual stream, loop input, short convolutions without activation, differential attention, routing by
+# sigmoid scores (csrc/stream_ops.hip, seq_mix.hip, diff_attn.hip, moe.hip)
+
+def gated_residual_norm(x, y=None, g=None, b=None, replace: bool = False, w=None, eps: float = 0.0, offset: float = 0.0,
+                        n32=None, h=None):
+    """The residual step of a pre-norm layer with gated sublayer outputs: x += y * sigmoid(g + b); with `replace`
+    x = y + b instead (a pass of a looped span starts from a projection plus a per-pass vector); y None: x as it is.
+    With `w`: n = x / sqrt(mean(x^2) + eps) * (offset + w) of the new x, to n32 (fp32) and / or h (activation type)."""
+    rows, n = x.shape
+    mode = 0 if y is None else (2 if replace else 1)
+    assert y is None or y.shape == (rows, n)
+    assert (mode == 1) == (g is not None) and (g is None or g.shape == (rows, n))
+    assert b is None or (b.numel() == n and b.is_contiguous())
+    assert (w is None) == (n32 is None and h is None) and (w is None or (w.numel() == n and w.is_contiguous()))
+    assert n32 is None or n32.shape == (rows, n)
+    assert h is None or h.shape == (rows, n)
+    nv.check("mv_gated_residual_norm", nv.lib().mv_gated_residual_norm(
+        None if y is None else _f32(y).data_ptr(), 0 if y is None else _ld(y),
+        None if g is None else _f32(g).data_ptr(), 0 if g is None else _ld(g),
+        None if b is None else _f32(b).data_ptr(), mode, _f32(x).data_ptr(), _ld(x),
+        None if w is None else _f32(w).data_ptr(), float(eps), float(offset),
+        None if n32 is None else _f32(n32).data_ptr(), 0 if n32 is None else _ld(n32),
+        None if h is None else h.data_ptr(), 0 if h is None else _ld(h), rows, n, 0 if h is None else _is_f32(h),
+        nv.stream_ptr()))
+
+
+def cast_concat(a, b, out):
+    """out = act([a | b]) for two fp32 operands of equal shape."""
+    rows, n = a.shape
+    assert b.shape == (rows, n) and out.shape == (rows, 2 * n)
+    nv.check("mv_cast_concat", nv.lib().mv_cast_concat(
+        _f32(a).data_ptr(), _ld(a), _f32(b).data_ptr(), _ld(b), out.data_ptr(), _ld(out), rows, n, _is_f32(out),
+        nv.stream_ptr()))
+
+
+def gelu_tanh(v, out):
+    rows, n = v.shape
+    assert out.shape == (rows, n)
+    nv.check("mv_gelu_tanh", nv.lib().mv_gelu_tanh(
+        _f32(v).data_ptr(), _ld(v), out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+def scale_(v, factor: float):
+    assert v.is_contiguous()
+    nv.check("mv_scale", nv.lib().mv_scale(_f32(v).data_ptr(), v.numel(), float(factor), nv.stream_ptr()))
+    return v
+
+
+def conv_taps(inp, state, w, step, out32=None, out_act=None, add_input: bool = False):
+    """y_t = (inp_t +) sum_j w[:, j] inp_(t - taps + 1 + j) per channel, no bias, no activation; inp [T, C] fp32,
+    state [slots, taps - 1, C] fp32 (the inputs before the step; updated), w [C, taps] fp32.  y goes to out32 (fp32)
+    and / or out_act (activation type)."""
+    tokens, ch = inp.shape
+    taps = w.shape[1]
+    assert w.shape == (ch, taps) and w.is_contiguous() and (out32 is not None or out_act is not None)
+    assert out32 is None or out32.shape == (tokens, ch)
+    assert out_act is None or out_act.shape == (tokens, ch)
+    assert state.is_contiguous() and state.shape[1:] == (max(taps - 1, 0), ch)
+    assert step.tokens == tokens and int(step.max_slot) < state.shape[0]
+    nv.check("mv_conv_taps", nv.lib().mv_conv_taps(
+        _f32(inp).data_ptr(), _ld(inp), _f32(state).data_ptr(), _f32(w).data_ptr(),
+        None if out32 is None else _f32(out32).data_ptr(), 0 if out32 is None else _ld(out32),
+        None if out_act is None else out_act.data_ptr(), 0 if out_act is None else _ld(out_act), int(add_input),
+        step.tok_row.data_ptr(), step.row_start.data_ptr(), step.row_len.data_ptr(), step.row_ctx.data_ptr(),
+        step.row_slot.data_ptr(), tokens, step.rows, ch, taps, 0 if out_act is None else _is_f32(out_act),
+        nv.stream_ptr()))
+
+
+def conv_qkv_store(qkv, state, w, q, k_cache, v_cache, step):
+    """The q | k | v columns of one projection (qkv [T, cq + ck + cv] fp32) through a causal convolution per channel
+    (w [cq + ck + cv, taps] fp32 and state [slots, taps - 1, cq + ck + cv]; w None: no convolution): queries to q
+    [T, cq] fp32, keys and values into the token's rows of k_cache [pages, page, ...ck] / v_cache [pages, page, ...cv]."""
+    tokens = qkv.shape[0]
+    page = k_cache.shape[1]
+    cq, ck, cv = q.shape[1], k_cache[0, 0].numel(), v_cache[0, 0].numel()
+    taps = 0 if w is None else w.shape[1]
+    assert qkv.shape[1] >= cq + ck + cv and q.shape[0] == tokens and step.tokens == tokens
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype
+    assert v_cache.shape[:2] == k_cache.shape[:2] and page == step.page and int(step.max_page) < k_cache.shape[0]
+    assert w is None or (w.shape == (cq + ck + cv, taps) and w.is_contiguous())
+    assert taps <= 1 or (state.is_contiguous() and state.shape[1:] == (taps - 1, cq + ck + cv)
+                         and int(step.max_slot) < state.shape[0])
+    nv.check("mv_conv_qkv_store", nv.lib().mv_conv_qkv_store(
+        _f32(qkv).data_ptr(), _ld(qkv), None if taps <= 1 else _f32(state).data_ptr(),
+        None if w is None else _f32(w).data_ptr(), _f32(q).data_ptr(), _ld(q), k_cache.data_ptr(), v_cache.data_ptr(),
+        step.tok_row.data_ptr(), step.tok_pos.data_ptr(), step.row_start.data_ptr(), step.row_len.data_ptr(),
+        step.row_ctx.data_ptr(), step.row_slot.data_ptr(), step.block_table.data_ptr(), step.block_table.stride(0), page,
+        tokens, step.rows, cq, ck, cv, taps, _is_f32(k_cache), nv.stream_ptr()))
+
+
+def diff_attn(q, k_cache, v_cache, out, gate, step, heads: int, kv_heads: int, d: int, dv: int, scale: float,
+              softcap: float, lam: float, out_scale: float, eps: float, tiled: bool = True):
+    """Differential attention: q [T, heads * 2 * d] fp32 (per head its two maps' queries), k_cache [pages, page,
+    kv_heads, 2 * d], v_cache [pages, page, kv_heads, dv]; causal softmax per map over the same values, o = a1 - lam a2,
+    out [T, heads * dv] = act(o / rms(o) * out_scale * sigmoid(gate[t, h])); gate [T, heads] fp32 or None.
+    `tiled`: rows of more than SCAN_SEQ_MAX tokens go to the matrix-core kernel where it applies."""
+    tokens = q.shape[0]
+    page = k_cache.shape[1]
+    assert q.shape[1] == heads * 2 * d and out.shape == (tokens, heads * dv) and out.dtype == k_cache.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert k_cache.shape[1:] == (page, kv_heads, 2 * d) and v_cache.shape == (k_cache.shape[0], page, kv_heads, dv)
+    assert gate is None or gate.shape == (tokens, heads)
+    assert int(step.max_page) < k_cache.shape[0] and page == step.page and step.tokens == tokens
+    chunks = step.n_chunks if tiled else 0
+    nv.check("mv_diff_attn", nv.lib().mv_diff_attn(
+        _f32(q).data_ptr(), _ld(q), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ld(out),
+        None if gate is None else _f32(gate).data_ptr(), 0 if gate is None else _ld(gate), step.tok_row.data_ptr(),
+        step.tok_pos.data_ptr(), step.block_table.data_ptr(), step.block_table.stride(0), page, tokens, heads, kv_heads,
+        d, dv, float(scale), float(softcap), float(lam), float(out_scale), float(eps), _is_f32(k_cache),
+        step.row_len.data_ptr(), step.ch_start.data_ptr() if chunks else None, step.ch_len.data_ptr() if chunks else None,
+        chunks, SCAN_SEQ_MAX, int(getattr(step, "short_tokens", -1)) if tiled else -1, nv.stream_ptr()))
+
+
+def moe_route_sigmoid(h, w_router, ids, weights):
+    """The `top` largest router outputs (fp32 logits of the activation-type input; ties to the lower index); the
+    weights are the sigmoids of the chosen outputs, not renormalised."""
+    tokens, n = h.shape
+    E, top = w_router.shape[0], ids.shape[1]
+    assert h.stride(1) == 1 and w_router.shape == (E, n) and w_router.is_contiguous()
+    assert ids.shape == (tokens, top) and weights.shape == (tokens, top) and ids.is_contiguous()
+    assert weights.is_contiguous() and ids.dtype == torch.int32
+    nv.check("mv_moe_route_sigmoid", nv.lib().mv_moe_route_sigmoid(
+        h.data_ptr(), _ld(h), _f32(w_router).data_ptr(), ids.data_ptr(), _f32(weights).data_ptr(), tokens, n, E, top,
+        _is_f32(h), nv.stream_ptr()))
+
+
+def gated_act_scaled(a, out, kind: int, scale, order=None, limit: float = 0.0, slope: float = 1.0):
+    """gated_act with both halves of row i multiplied by scale[order[i]] (order None: scale[i]) first."""
+    rows, n = out.shape
+    assert a.shape == (rows, 2 * n) and scale.is_contiguous() and (order is None or order.numel() == rows)
+    assert scale.numel() >= rows
+    nv.check("mv_gated_act_scaled", nv.lib().mv_gated_act_scaled(
+        _f32(a).data_ptr(), _ld(a), out.data_ptr(), _ld(out), rows, n, int(kind), float(limit), float(slope),
+        _f32(scale).data_ptr(), None if order is None else _i32(order).data_ptr(), _is_f32(out), nv.stream_ptr()))

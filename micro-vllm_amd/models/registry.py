@@ -6,7 +6,7 @@ A family = (configuration reader, model object, runner and cache manager the eng
              ModelGraphRunner / KVCacheManager);
   "ragged" - stacks with an fp32 residual stream whose layers are listed one by one (recurrent
              mixers, windowed or latent attention, dense or routed feed-forwards), run step by step
-             over ragged batches (RaggedRunner / HybridCacheManager): Pagazen, Fagunex, Nesisun.
+             over ragged batches (RaggedRunner / HybridCacheManager): Pagazen, Fagunex, Nesisun, Solopel.
 """
 from typing import Callable, Dict
 
@@ -45,9 +45,19 @@ def _load_nesisun(config_json, files, name):
     return NesisunModel(cfg, files)
 
 
+def _load_solopel(config_json, files, name):
+    from .solopel import SolopelConfig, SolopelModel, tensor_shapes
+    cfg = SolopelConfig.from_json(config_json, name)
+    for tensor, shape in tensor_shapes(cfg).items():
+        if tensor not in files:
+            raise KeyError(f"tensor {tensor!r} {shape} is not in the checkpoint")
+    return SolopelModel(cfg, files)
+
+
 register("Pagazen", _load_pagazen)
 register("Fagunex", _load_fagunex)
 register("Nesisun", _load_nesisun)
+register("Solopel", _load_solopel)
 
 
 def loader_for(config_json: dict):
