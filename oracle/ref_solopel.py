@@ -49,40 +49,35 @@ def softmax_rows(s):
     return e / e.sum()
 
 
+def latent_attention(q, c, uk, uv, scale):
+    """q [T, H, d]; c [T, R] the normed latents; uk [H*d, R], uv [H*dv, R]: causal softmax per head over the keys
+    uk_h c_j, values uv_h c_j."""
+    T, H, d = q.shape
+    k = (c @ uk.T).view(T, H, d)
+    v = (c @ uv.T).view(T, H, -1)
+    out = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for hd in range(H):
+        for i in range(T):
+            s = (k[:i + 1, hd] @ q[i, hd]) * scale
+            out[i, hd] = softmax_rows(s) @ v[:i + 1, hd]
+    return out
+
+
 def latent_mixer(h, W, p, m, eps):
     """Keys and values of every head come from ONE normed latent per token; no positions enter."""
-    H, d, dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+    H, d = int(m["heads"]), int(m["dim"])
     T = h.shape[0]
     q = (h @ W[p + "q"].T).view(T, H, d)
     c = rms_unit(h @ W[p + "dkv"].T, eps) * W[p + "dkv.norm"]
-    k = (c @ W[p + "uk"].T).view(T, H, d)
-    v = (c @ W[p + "uv"].T).view(T, H, dv)
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
-    for hd in range(H):
-        for i in range(T):
-            s = (k[:i + 1, hd] @ q[i, hd]) * float(m["scale"])
-            out[i, hd] = softmax_rows(s) @ v[:i + 1, hd]
-    return out.reshape(T, H * dv) @ W[p + "o"].T
+    return latent_attention(q, c, W[p + "uk"], W[p + "uv"], float(m["scale"])).reshape(T, -1) @ W[p + "o"].T
 
 
-def difference_mixer(h, W, p, m, eps):
-    """Two attention maps per head over the same values; o = a1 - lambda a2, unit-normed per head, times
-    (1 - diff), times a sigmoid gate of one number per head."""
-    H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
-    T = h.shape[0]
-    diff, scale = float(m["diff"]), float(m["scale"])
-    cap = float(m["softcap"]) if m.get("softcap") else 0.0
-
-    def proj(name):
-        u = h @ W[p + name].T
-        return causal_conv(u, W[p + name + ".conv"]) if (p + name + ".conv") in W else u
-
-    q = proj("q").view(T, H, 2, d)
-    k = proj("k").view(T, G, 2, d)
-    v = proj("v").view(T, G, dv)
-    lam = math.exp(float((W[p + "lq1"] * W[p + "lk1"]).sum())) - math.exp(float((W[p + "lq2"] * W[p + "lk2"]).sum())) + diff
-    gate = torch.sigmoid(h @ W[p + "g"].T)            # [T, H]
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
+def difference_attention(q, k, v, gate, scale, cap, lam, diff, eps):
+    """q [T, H, 2, d], k [T, G, 2, d], v [T, G, dv], gate [T, H] (logits) or None: two causal softmax maps per head
+    over the same values; o = a1 - lam a2, unit-normed over the head, times (1 - diff), times sigmoid(gate)."""
+    T, H = q.shape[:2]
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
     for hd in range(H):
         g = hd // (H // G)
         for i in range(T):
@@ -92,8 +87,28 @@ def difference_mixer(h, W, p, m, eps):
                 if cap:
                     s = cap * torch.tanh(s / cap)
                 a.append(softmax_rows(s) @ v[:i + 1, g])
-            o = a[0] - lam * a[1]
-            out[i, hd] = rms_unit(o, eps) * (1.0 - diff) * gate[i, hd]
+            o = rms_unit(a[0] - lam * a[1], eps) * (1.0 - diff)
+            out[i, hd] = o if gate is None else o * torch.sigmoid(gate[i, hd])
+    return out
+
+
+def difference_lambda(W, p, diff):
+    return math.exp(float((W[p + "lq1"] * W[p + "lk1"]).sum())) - math.exp(float((W[p + "lq2"] * W[p + "lk2"]).sum())) + diff
+
+
+def difference_mixer(h, W, p, m, eps):
+    """Projections, a short causal convolution behind each of q, k, v, then the two-map attention."""
+    H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+    T = h.shape[0]
+    diff = float(m["diff"])
+
+    def proj(name):
+        u = h @ W[p + name].T
+        return causal_conv(u, W[p + name + ".conv"]) if (p + name + ".conv") in W else u
+
+    out = difference_attention(proj("q").view(T, H, 2, d), proj("k").view(T, G, 2, d), proj("v").view(T, G, dv),
+                               h @ W[p + "g"].T, float(m["scale"]), float(m["softcap"]) if m.get("softcap") else 0.0,
+                               difference_lambda(W, p, diff), diff, eps)
     return out.reshape(T, H * dv) @ W[p + "o"].T
 
 
