@@ -300,7 +300,7 @@ class RaggedRunner:
     def cache_layout(self):
         """(kv_layers, state_layers) for HybridCacheManager: what every layer RUN keeps per sequence."""
         kv, state = {}, {}
-        if self.gated_prenorm:
+        if self.cfg.architecture == "Solopel":
             for i, (_, layer) in enumerate(self.runs):
                 m = layer["mixer"]
                 state[i] = {"canon": (self.cfg.taps - 1, self.width)} if self.cfg.taps else {}

@@ -75,7 +75,7 @@ def test_cache_layout_gives_every_layer_run_its_own_pages_and_tails(mv):
     from micro_vllm_amd.core.layer.ragged_runner import RaggedRunner
     cfg = config_a()
     runner = RaggedRunner.__new__(RaggedRunner)
-    runner.cfg, runner.width, runner.runs, runner.gated_prenorm = cfg, cfg.width, cfg.layer_runs(), True
+    runner.cfg, runner.width, runner.runs = cfg, cfg.width, cfg.layer_runs()
     kv, state = runner.cache_layout()
     assert sorted(kv) == list(range(11)) and sorted(state) == list(range(11))
     assert kv[0] == (2, 48, 40) and kv[1] == kv[4] == kv[7] == (1, 72, 0) and kv[2] == kv[5] == (1, 32, 72)
