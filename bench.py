@@ -87,6 +87,14 @@ def parse():
                          "model of equal width, depth and feed-forward parameters; one JSON line of its own")
     ap.add_argument("--nesisun-widths", default="1024,2048,4096")
     ap.add_argument("--nesisun-kernels", action="store_true", help="with --nesisun: per-op times of one step on stderr")
+    ap.add_argument("--solopel", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the Solopel design "
+                         "(gated pre-norm layers, latent attention without positions, differential attention, dense "
+                         "and routed feed-forwards, a looped span; random weights) at a few widths, with every "
+                         "feed-forward routed and with dense ones only, beside Fagunex - the family's other design "
+                         "with latent attention and routed experts - at equal width and depth; one JSON line of its own")
+    ap.add_argument("--solopel-widths", default="1024,2048,4096")
+    ap.add_argument("--solopel-kernels", action="store_true", help="with --solopel: per-op times of one step on stderr")
     return ap.parse_args()
 
 
@@ -729,6 +737,35 @@ def nesisun_compare(args, dev):
                       "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
 
 
+def solopel_compare(args, dev):
+    """Prefill (one prompt of --ctx tokens) and decode (bs 1 and 8 at context --ctx) of the Solopel design through
+    InferenceEngine.run_ragged - once with every feed-forward routed (8 experts of which 2 are used plus a shared one,
+    4 x width active), once with dense ones of 4 x width - beside Fagunex with attention in every layer and the same
+    routed feed-forward.  Random weights, 4 layers, vocabulary 32000, 128-wide heads, latents of 512.  Solopel: three
+    latent-attention layers and one differential attention (two 64-wide maps per head, one key/value head per four
+    query heads), all causal, the span of four layers entered once through the loop's input projection; Fagunex: two
+    windowed (1024) and two causal latent attentions with a 64-wide rotated key part."""
+    import micro_vllm_amd  # noqa: F401
+    from micro_vllm_amd.core.engine import InferenceEngine
+    from micro_vllm_amd.models import fagunex, solopel
+
+    S, layers, rows = args.ctx, 4, []
+    for width in [int(w) for w in args.solopel_widths.split(",")]:
+        row = {"width": width, "layers": layers, "ctx": S}
+        for name, mod, cfg in (("solopel_routed", solopel, solopel.bench_config(width, layers, moe_every=1)),
+                               ("solopel_dense", solopel, solopel.bench_config(width, layers, moe_every=0)),
+                               ("fagunex", fagunex, fagunex.bench_config(width, layers, every=1))):
+            eng = InferenceEngine(model=mod.build_random_model(cfg, seed=1), max_batch_size=8, max_prefill_tokens=S,
+                                  n_blocks=9 * (S // 64 + 4), max_tokens=S + 256, state_slots=9)
+            row.update(_ragged_engine_row(eng, cfg, S, name, args.solopel_kernels, width))
+            del eng
+            torch.cuda.empty_cache()
+        log(f"[bench] {row}")
+        rows.append(row)
+    print(json.dumps({"metric": "Solopel beside Fagunex (ragged family): prefill and decode tokens/s at equal size",
+                      "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
+
+
 def pagazen_kernel_table(eng, ids, width):
     """Per-op time of one prefill step and one single-token step (rocprof-free: HIP events around each
     wrapper call), printed on stderr."""
@@ -740,7 +777,8 @@ def pagazen_kernel_table(eng, ids, width):
              "dyt_shift", "dyt_gather", "dyt_residual", "unitnorm_residual", "rmsnorm_rows", "gelu_gate_rows", "silu_mul",
              "sigmoid_gate", "linear_heads", "linear_segments", "gate_lower_bound_", "scan_gated", "latent_prep",
              "latent_attn", "moe_route", "moe_plan", "moe_combine", "embed_pair", "add_rmsnorm", "rmsnorm_gather",
-             "gated_act", "qk_rotary_store", "moe_route_scored"]
+             "gated_act", "qk_rotary_store", "moe_route_scored", "gated_residual_norm", "cast_concat", "gelu_tanh",
+             "scale_", "conv_taps", "conv_qkv_store", "diff_attn", "moe_route_sigmoid", "gated_act_scaled"]
     saved = {n: getattr(ops, n) for n in names}
     saved_call = ops.AnyLinear.__call__
 
@@ -875,6 +913,9 @@ def main():
     if args.nesisun:
         assert world == 1, "--nesisun runs on one GPU"
         return nesisun_compare(args, dev)
+    if args.solopel:
+        assert world == 1, "--solopel runs on one GPU"
+        return solopel_compare(args, dev)
     peers = world > 1                 # ranks to synchronise with
     if args.as_rank_of:
         assert world == 1, "--as-rank-of runs one process"

@@ -673,7 +673,7 @@ int mv_latent_prep(const float* dkv, int64_t ldkv, const float* w_norm, float ep
 /* out[t, h*rank ..] = sum_j softmax_j( q_abs[t,h] . cache[j] * scale ) cache[j][:rank] over the keys j <= position
  * (window > 0: only the last `window` of them); sinks != NULL: exp(sinks[h]) joins the denominator.
  * chunks > 0: rows of more than max_len tokens, cut into chunks of up to 64 (ch_start / ch_len), run on the matrix
- * cores where the shape allows it (bf16, pages of 64, rank in {64,128,256,512}, r in {32,64}): q . k in bf16 (q
+ * cores where the shape allows it (bf16, pages of 64, rank in {64,128,256,512}, r in {0,32,64}): q . k in bf16 (q
  * rounded as the cached latents are), softmax in fp32, P . V with fp32 P; every other token takes the
  * one-workgroup-per-(token, head group) form. */
 int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out, int64_t ldo, const int32_t* tok_row,

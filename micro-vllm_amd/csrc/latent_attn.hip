@@ -427,7 +427,7 @@ static int launch_latent_tile(const float* q, int64_t ldq, const void* cache, vo
 
 // the (latent width, rotated width) pairs the tile kernel is built for
 static bool latent_tile_shape(int R, int r) {
-    return (r == 32 || r == 64) && (R == 64 || R == 128 || R == 256 || R == 512) && (R + r) % 32 == 0;
+    return (r == 0 || r == 32 || r == 64) && (R == 64 || R == 128 || R == 256 || R == 512) && (R + r) % 32 == 0;
 }
 
 }  // namespace mv
@@ -475,7 +475,7 @@ int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out
     if (rank == R_ && r == r_)                                                                                     \
         rc = launch_latent_tile<(R_ + r_) / 32, R_ / 16>(q_abs, ldq, cache, out, ldo, pr, ch_start, ch_len, chunks, \
                                                           sinks, heads, scale, window, s);
-        MV_LT(64, 32) MV_LT(64, 64) MV_LT(128, 32) MV_LT(128, 64) MV_LT(256, 32) MV_LT(256, 64) MV_LT(512, 32) MV_LT(512, 64)
+        MV_LT(64, 0) MV_LT(128, 0) MV_LT(256, 0) MV_LT(512, 0) MV_LT(64, 32) MV_LT(64, 64) MV_LT(128, 32) MV_LT(128, 64) MV_LT(256, 32) MV_LT(256, 64) MV_LT(512, 32) MV_LT(512, 64)
 #undef MV_LT
         if (rc != MV_OK) return rc;
         plain_max = max_len;
