@@ -120,7 +120,7 @@ class RaggedRunner:
             self.pair_embed = self._act(model.get("bigram"))
         elif self.gated_prenorm:
             self.final_norm = self._small(model.get("final.norm"))
-            if cfg.loop:
+            if cfg.looped:
                 self.loop_in = self._linear(model.get("loop.in"))
                 self.loop_step = self._small(model.get("loop.step"))
         else:
@@ -466,7 +466,8 @@ class RaggedRunner:
 
     def _run(self, step: RaggedStep, cache: HybridCacheManager, want, residuals) -> torch.Tensor:
         cfg, T = self.cfg, step.tokens
-        x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
+        if not self.gated_prenorm:       # that design's stack lays out its own streams
+            x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
         if self.parallel_prenorm:
             ops.embed_pair(self.embed, self.pair_embed, step.ids, step.tok_prev, x, cfg.embed_scale, cfg.pair_buckets,
                            cfg.pair_mul_prev, cfg.pair_mul_cur, w=self._w[self.runs[0][0]]["norm1"], eps=cfg.eps, h=h)

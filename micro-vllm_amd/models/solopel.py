@@ -65,13 +65,18 @@ class SolopelConfig:
     def run_plan(self):
         """[(layer, number of the loop pass that STARTS with this run, or -1)] in running order."""
         n = len(self.layers)
-        if not self.loop:
+        if not self.looped:
             return [(i, -1) for i in range(n)]
         a, b, times = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
         plan = [(i, -1) for i in range(a)]
         for t in range(times):
             plan += [(i, t if i == a else -1) for i in range(a, b)]
         return plan + [(i, -1) for i in range(b, n)]
+
+    @property
+    def looped(self) -> bool:
+        """Whether a span of at least one layer is looped (an empty span has no pass and needs no tensors)."""
+        return bool(self.loop) and int(self.loop["start"]) < int(self.loop["stop"])
 
     def layer_runs(self):
         """[(index of the layer whose tensors the run uses, its description)] in running order."""
@@ -92,7 +97,7 @@ class SolopelConfig:
         loop = d.get("loop")
         if loop:
             a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
-            if not (0 <= a < b <= len(layers)) or times < 1:
+            if not (0 <= a <= b <= len(layers)) or times < 1:
                 raise ValueError(f"loop {loop!r} does not fit {len(layers)} layers")
         canon = d.get("canon")
         return cls(vocab_size=int(d["vocab"]), width=int(d["width"]), layers=layers, eps=float(d["norm"]["eps"]),
@@ -117,7 +122,7 @@ def tensor_shapes(cfg: SolopelConfig) -> Dict[str, tuple]:
     """Name -> shape of every tensor a checkpoint of this configuration holds."""
     W = cfg.width
     out = {"embed": (cfg.vocab_size, W), "final.norm": (W,)}
-    if cfg.loop:
+    if cfg.looped:
         out.update({"loop.in": (W, 2 * W), "loop.step": (int(cfg.loop["times"]), W)})
     for i, layer in enumerate(cfg.layers):
         p, m = f"l{i}.", layer["mixer"]
@@ -203,7 +208,7 @@ def bench_config(width: int, n_layers: int, vocab: int = 32000, ff_mult: int = 4
     for i in range(n_layers):
         mlp = moe if moe_every and i % moe_every == moe_every - 1 else dense
         if i % every == every - 1:
-            mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 128, "conv": 4, "diff": 0.3,
+            mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 128, "conv": 4, "diff": 0.2,
                      "scale": 64 ** -0.5, "softcap": 30.0}
             layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
         else:

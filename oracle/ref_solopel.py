@@ -171,7 +171,7 @@ def forward(config, weights, tokens, dtype=torch.float64, residuals=None):
                 residuals.append(x.clone())
 
     loop = config.get("loop")
-    if loop:
+    if loop and int(loop["start"]) < int(loop["stop"]):
         a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
         run(range(a))
         for t in range(times):

@@ -53,7 +53,7 @@ def config_b():
     one expert used, a single expert, one tap, no convolution behind the projections, no soft cap, no loop, unit logit
     scale; widths the wave-tile projections and the matrix-core attention take (so the bf16 run uses both)."""
     return SolopelConfig(vocab_size=256, width=128, eps=1e-6, taps=1, logit_scale=1.0, loop=None, layers=[
-        layer("attention", differential(heads=2, kv_heads=2, dim=64, vdim=64, conv=0, diff=0.3, scale=0.125, softcap=0),
+        layer("attention", differential(heads=2, kv_heads=2, dim=64, vdim=64, conv=0, diff=0.25, scale=0.125, softcap=0),
               moe(experts=4, top=1, ff=64, shared=64)),
         layer("latent_attention", latent(heads=2, dim=64, vdim=64, rank=64, scale=0.125), dense(128)),
         layer("attention", differential(heads=4, kv_heads=1, dim=32, vdim=64, conv=1, diff=0.5, scale=0.2, softcap=30.0),
@@ -95,7 +95,7 @@ def random_config(seed):
                                                             rng.choice([0.1, 0.2, 0.5])), mlp))
         else:
             kv = rng.choice([1, 2, 3])
-            dim, vdim = rng.choice([(8, 8), (24, 40), (32, 32), (32, 64), (64, 64), (64, 128), (48, 96), (128, 128), (40, 200)])
+            dim, vdim = rng.choice([(8, 8), (24, 40), (32, 32), (32, 64), (64, 64), (64, 128), (56, 72), (128, 128), (40, 200)])
             layers.append(layer("attention", differential(kv * rng.choice([1, 2, 4]), kv, dim, vdim, rng.choice([0, 1, 2, 4, 5]),
                                                           rng.choice([0.1, 0.3, 0.8]), rng.choice([0.1, dim ** -0.5, 0.5]),
                                                           rng.choice([0, 2.0, 20.0, 50.0])), mlp))

@@ -190,7 +190,7 @@ def diff_case(ops, H, G, d, dv, dt, portions, q, k, v, gate, scale, cap, lam, di
     return torch.cat(outs).view(T, H, dv)
 
 
-SHAPES = [(6, 2, 24, 40), (4, 4, 48, 96), (2, 1, 64, 64), (4, 1, 32, 64), (2, 2, 64, 128), (3, 3, 32, 32),
+SHAPES = [(6, 2, 24, 40), (4, 2, 56, 72), (2, 1, 64, 64), (4, 1, 32, 64), (2, 2, 64, 128), (3, 3, 32, 32),
           (2, 1, 128, 128), (1, 1, 8, 200)]
 
 

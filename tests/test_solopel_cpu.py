@@ -40,11 +40,15 @@ def test_config_reader_run_plan_and_tensor_table(mv):
     assert "l0.canon1" not in tensor_shapes(config_c())
     for spoil in (lambda d: d["layers"][0].update(type="conv"), lambda d: d["layers"][0]["mlp"].update(kind="glu"),
                   lambda d: d["layers"][0]["mixer"].update(kv_heads=4), lambda d: d["loop"].update(stop=9),
-                  lambda d: d["loop"].update(times=0), lambda d: d["loop"].update(start=4, stop=4)):
+                  lambda d: d["loop"].update(times=0), lambda d: d["loop"].update(start=4, stop=3)):
         bad = json.loads(json.dumps(cfg.to_json()))
         spoil(bad)
         with pytest.raises(ValueError):
             SolopelConfig.from_json(bad)
+    empty = json.loads(json.dumps(cfg.to_json()))
+    empty["loop"].update(start=2, stop=2)                       # an empty span: no pass, no loop tensors
+    e = SolopelConfig.from_json(empty)
+    assert e.runs == [0, 1, 2, 3, 4] and "loop.in" not in tensor_shapes(e)
     for seed in range(20):
         c = random_config(seed)
         assert SolopelConfig.from_json(json.loads(json.dumps(c.to_json()))).to_json() == c.to_json()
