@@ -283,7 +283,8 @@ def test_soft_cap_flattens_large_scores(ops, f32):
 
 
 # ----------------------------------------------------------------------------------------------- latent attention
-@pytest.mark.parametrize("H,d,dv,R", [(3, 40, 24, 72), (2, 64, 64, 64), (4, 32, 48, 128), (1, 16, 16, 33)])
+@pytest.mark.parametrize("H,d,dv,R", [(3, 40, 24, 72), (2, 64, 64, 64), (4, 32, 48, 128), (1, 16, 16, 33), (2, 32, 40, 256),
+                                      (1, 64, 32, 512)])
 @pytest.mark.parametrize("f32", [False, True])
 def test_latent_attention_without_positions(ops, H, d, dv, R, f32):
     """The product path's sequence (latent into the page, queries carried into the latent space per head, attention
